@@ -1,0 +1,244 @@
+/*
+ * moe_mi355.h -- C ABI of libmoe_mi355.so: the MoE-layer hot path of MoE-Gen
+ * (router -> dispatch -> grouped SwiGLU experts -> weighted combine, plus
+ * expert-weight staging) as hand-written HIP kernels for one MI355X (gfx950).
+ *
+ * Conventions
+ *   - every pointer marked "device" is HBM memory owned by the caller; the
+ *     library allocates nothing inside the compute entry points;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *     all work is enqueued on it and the call returns without synchronising;
+ *   - return value 0 on success, a negative moe_status otherwise; the message
+ *     of the last failure on the calling thread is moe_last_error();
+ *   - bf16 tensors are raw 16-bit patterns, fp8 tensors are OCP e4m3fn bytes
+ *     (torch.float8_e4m3fn), both row-major with the last dimension contiguous.
+ *
+ * Reference paths are relative to the EfficientMoE/MoE-Gen checkout.
+ */
+#ifndef MOE_MI355_H
+#define MOE_MI355_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum moe_status {
+    MOE_OK = 0,
+    MOE_ERR_INVALID = -1,    /* bad argument / unsupported shape */
+    MOE_ERR_WORKSPACE = -2,  /* workspace too small */
+    MOE_ERR_HIP = -3,        /* a HIP runtime call failed */
+    MOE_ERR_STATE = -4       /* stager used out of protocol */
+} moe_status;
+
+/* Message of the most recent failure on this thread ("" if none). */
+const char* moe_last_error(void);
+
+/* Library version string. */
+const char* moe_version(void);
+
+/* ---------------------------------------------------------------- router */
+
+enum { MOE_SCORE_SOFTMAX = 0, MOE_SCORE_SIGMOID = 1 };
+enum { MOE_TOPK_GREEDY = 0, MOE_TOPK_GROUP_LIMITED_GREEDY = 1, MOE_TOPK_NOAUX_TC = 2 };
+enum { MOE_SCALE_NEVER = 0, MOE_SCALE_IF_NOT_NORM = 1, MOE_SCALE_ALWAYS = 2 };
+
+typedef struct moe_router_params {
+    int32_t n_tokens;        /* n */
+    int32_t hidden;          /* h, multiple of 8 */
+    int32_t n_experts;       /* E <= 256 */
+    int32_t top_k;           /* k <= 16, k <= E */
+    int32_t n_group;         /* G (1 for greedy); E % G == 0, G <= 32 */
+    int32_t topk_group;      /* groups kept */
+    int32_t scoring;         /* MOE_SCORE_* */
+    int32_t method;          /* MOE_TOPK_* */
+    int32_t norm_topk_prob;  /* renormalise the k weights to sum 1 (only if k > 1) */
+    int32_t scale_mode;      /* MOE_SCALE_* : V2 scales only when not normalising
+                                (modeling_deepseek_v2.py:529-533), V3 always
+                                (modeling_deepseek_v3.py:554-559) */
+    int32_t logits_bf16;     /* round logits to bf16 before scoring (Mixtral's bf16 gate) */
+    int32_t weights_bf16;    /* round the final weights to bf16 values (Mixtral) */
+    float norm_eps;          /* added to the sum before dividing: 1e-20 DeepSeek, 0 Mixtral */
+    float routed_scaling_factor;
+} moe_router_params;
+
+/*
+ * Fused router: replaces MoEGate.forward (modeling_deepseek_v3.py:500-561,
+ * modeling_deepseek_v2.py:483-533) and the routing lines of
+ * MixtralSparseMoeBlock.forward (transformers 4.42.0).  One kernel computes the
+ * fp32 logits x @ W^T, the scores (softmax, or sigmoid + e_score_correction_bias),
+ * the group-limited selection, top-k (descending score, ties to the lower expert
+ * index), renormalisation and routed scaling.
+ *   x          device bf16 [n, h]
+ *   w_gate     device bf16 [E, h]
+ *   bias       device fp32 [E] (e_score_correction_bias) or NULL
+ *   topk_idx   device int32 [n, k]   out
+ *   topk_w     device fp32 [n, k]    out
+ *   logits_out device fp32 [n, E]    out, may be NULL
+ */
+int moe_router(const void* x, const void* w_gate, const float* bias,
+               const moe_router_params* params, int32_t* topk_idx, float* topk_w,
+               float* logits_out, void* stream);
+
+/* -------------------------------------------------------------- dispatch */
+
+/*
+ * Replaces the first half of moe_infer (modeling_deepseek_v3.py:630-634,673 ==
+ * modeling_deepseek_v2.py:672-676,715): per-expert histogram, exclusive prefix
+ * sum and the stable sort of the flat (token*k + slot) list by expert id, then
+ * (optionally) the row gather sorted_tokens = x[idxs // k].  No host sync.
+ *   topk_idx  device int32 [n, k]
+ *   counts    device int32 [E]      out  tokens per expert
+ *   offsets   device int32 [E+1]    out  exclusive prefix sum of counts
+ *   perm      device int32 [n*k]    out  perm[r] = flat index at sorted row r
+ *   pos       device int32 [n*k]    out  pos[flat] = sorted row (inverse of perm)
+ *   x         device bf16 [n, h]         may be NULL together with xs
+ *   xs        device bf16 [n*k, h]  out  gathered rows, may be NULL
+ *   workspace device, at least moe_dispatch_workspace_bytes(n, k, E) bytes
+ */
+size_t moe_dispatch_workspace_bytes(int32_t n_tokens, int32_t top_k, int32_t n_experts);
+int moe_dispatch(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k, int32_t n_experts,
+                 int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* pos,
+                 const void* x, int32_t hidden, void* xs,
+                 void* workspace, size_t workspace_bytes, void* stream);
+
+/* ----------------------------------------------------- grouped SwiGLU GEMM */
+
+/*
+ * Replaces the expert loop of moe_infer (modeling_deepseek_v3.py:675-691) with
+ * Expert_Wrapper.forward (Wrapper.py:470-530) and DeepseekV3MLP.forward
+ * (:463-467; V2 :449-453; Mixtral w2(silu(w1 x) * w3 x)) for ALL experts in two
+ * launches: for expert e and its rows r in [offsets[e], offsets[e+1])
+ *     a[r] = bf16( bf16(silu(bf16(x_r Wg_e^T))) * bf16(x_r Wu_e^T) )
+ *     y[r] = bf16( a[r] Wd_e^T )
+ * on bf16 MFMA with fp32 accumulation.
+ *   x         device bf16: rows of the sorted token matrix [n_rows, h]; or, when
+ *             row_map != NULL, the unsorted matrix, row r being x[row_map[r]]
+ *   row_map   device int32 [n_rows] or NULL
+ *   w_gate/w_up/w_down   device arrays of E device pointers: Wg_e, Wu_e bf16
+ *             [I, h]; Wd_e bf16 [h, I]  (nn.Linear [out, in] layout)
+ *   offsets   device int32 [E+1] (as written by moe_dispatch); offsets[E] <= n_rows
+ *   act       device bf16 [n_rows, I]  scratch for a
+ *   y         device bf16 [n_rows, h]  out
+ *   workspace device, at least moe_grouped_workspace_bytes(n_rows, E) bytes
+ * Requires h % 64 == 0 and I % 64 == 0.
+ */
+size_t moe_grouped_workspace_bytes(int32_t n_rows, int32_t n_experts);
+int moe_grouped_swiglu_bf16(const void* x, const int32_t* row_map,
+                            const void* const* w_gate, const void* const* w_up,
+                            const void* const* w_down, const int32_t* offsets,
+                            int32_t n_rows, int32_t n_experts, int32_t hidden, int32_t inter,
+                            void* act, void* y, void* workspace, size_t workspace_bytes,
+                            void* stream);
+
+/*
+ * W8A16 variant: weights are fp8 e4m3fn with one fp32 scale per 128x128 block;
+ * each weight element is dequantised in registers as bf16(f32(q) * scale)
+ * (deepseek_v3_dequantization, Wrapper.py:109-138) before it reaches the MFMA.
+ *   s_gate/s_up  device arrays of E pointers to fp32 [ceil(I/128), ceil(h/128)]
+ *   s_down       device array  of E pointers to fp32 [ceil(h/128), ceil(I/128)]
+ * Requires h % 128 == 0 and I % 128 == 0.
+ */
+int moe_grouped_swiglu_w8a16(const void* x, const int32_t* row_map,
+                             const void* const* w_gate, const void* const* w_up,
+                             const void* const* w_down,
+                             const float* const* s_gate, const float* const* s_up,
+                             const float* const* s_down, const int32_t* offsets,
+                             int32_t n_rows, int32_t n_experts, int32_t hidden, int32_t inter,
+                             void* act, void* y, void* workspace, size_t workspace_bytes,
+                             void* stream);
+
+/*
+ * Stand-alone block dequantisation (Wrapper.py:109-138), used by tests and by
+ * callers that want a bf16 copy:  out = bf16(f32(q) * scale[i/128, j/128]).
+ *   q device fp8 [rows, cols]; scale device fp32 [ceil(rows/128), ceil(cols/128)];
+ *   out device bf16 [rows, cols].
+ */
+int moe_dequant_fp8_block128(const void* q, const float* scale, int32_t rows, int32_t cols,
+                             void* out, void* stream);
+
+/* --------------------------------------------------------------- combine */
+
+enum {
+    MOE_COMBINE_F32 = 0,       /* V3: fp32 products and sum, one rounding (modeling_deepseek_v3.py:702-710) */
+    MOE_COMBINE_BF16_PROD = 1, /* V2: bf16 weight, bf16 products, fp32-accumulated sum (modeling_deepseek_v2.py:744-757) */
+    MOE_COMBINE_BF16_SEQ = 2   /* Mixtral: bf16 accumulator, experts in ascending id (index_add_) */
+};
+
+/*
+ * Replaces the second half of moe_infer (inverse permutation + weighted sum over
+ * the k slots) and the shared-expert add (modeling_deepseek_v3.py:624-625):
+ *     out[t] = sum_j w[t,j] * y[pos[t*k+j]]   (+ shared[t])
+ *   y        device bf16 [n*k, h]   expert outputs in sorted-row order
+ *   pos      device int32 [n*k]
+ *   topk_idx device int32 [n, k]    (needed by MOE_COMBINE_BF16_SEQ only; else may be NULL)
+ *   topk_w   device fp32 [n, k]
+ *   shared   device bf16 [n, h] or NULL
+ *   out      device bf16 [n, h]
+ */
+int moe_combine(const void* y, const int32_t* pos, const int32_t* topk_idx, const float* topk_w,
+                const void* shared, int32_t n_tokens, int32_t top_k, int32_t hidden,
+                int32_t mode, void* out, void* stream);
+
+/* ------------------------------------------------- expert-weight staging */
+
+/*
+ * Slot pool + cyclic prefetch of whole expert modules from pinned host memory
+ * into HBM slots on a private copy stream.  Replaces, for the weights half,
+ * HtoD_Engine::HtoD_Worker (core/HtoD_Engine/HtoD_Engine.cpp:201-268),
+ * GPU_Weight_Buffer::{acquireEmptyBuffer, get_weights, releaseBuffer,
+ * weights_copy_complete, clear_expert_buffer}
+ * (core/GPU_Weight_Buffer/GPU_Weight_Buffer.cpp:146-308) and
+ * Weights_Storage::get_module_weights_storage (core/Weights_Storage/Weights_Storage.cpp:80).
+ * The reference hands slots over through a host condition variable after a
+ * stream synchronise; here hand-off is by events: acquire() makes the caller's
+ * compute stream wait for the copy, release() makes the next copy into the slot
+ * wait for the compute stream.  The host never blocks.
+ *
+ * A "module type" is a family of modules sharing one slot shape (the reference's
+ * "routed_expert", "shared_expert").  Modules are copied in the cyclic order in
+ * which they were added, routing-agnostically, whenever a slot of their type is
+ * free -- the policy of the reference's worker loop.
+ */
+typedef struct moe_stager moe_stager;
+
+enum { MOE_STAGE_DEVICE = 0,       /* slots are device memory, copies use hipMemcpyAsync */
+       MOE_STAGE_HOST_MEMCPY = 1   /* slots are host memory, copies use memcpy: host-only tests */ };
+
+/* n_types module types; slot_bytes[t] bytes per slot; n_slots[t] slots;
+ * slot_mem[t] points to n_slots[t]*slot_bytes[t] bytes owned by the caller. */
+int moe_stage_create(moe_stager** out, int32_t n_types, const size_t* slot_bytes,
+                     const int32_t* n_slots, void* const* slot_mem, int32_t backend);
+/* Register a module: n_tensors source ranges (pinned host pointers) copied back
+ * to back into the slot at dst_offsets.  Returns the module id (>= 0). */
+int moe_stage_add_module(moe_stager* s, int32_t type, int32_t n_tensors,
+                         const void* const* src, const size_t* bytes, const size_t* dst_offsets);
+/* Issue copies for the next modules of every type while free slots exist
+ * (one turn of the reference's worker loop per free slot).  Returns the number
+ * of modules whose copy was enqueued. */
+int moe_stage_pump(moe_stager* s);
+/* get_weights: make `stream` wait until module `id` is resident; *slot receives
+ * its slot index.  If the module is not yet scheduled, pumps until it is; fails
+ * with MOE_ERR_STATE if no slot can become free (all slots held). */
+int moe_stage_acquire(moe_stager* s, int32_t id, void* stream, int32_t* slot);
+/* free_weights_buffer: the slot may be overwritten once `stream` reaches this point. */
+int moe_stage_release(moe_stager* s, int32_t id, void* stream);
+/* Whether module `id` currently occupies a slot (copied or copy in flight). */
+int moe_stage_resident(moe_stager* s, int32_t id);
+/* Grow (or shrink back) the number of usable slots of a type within the memory
+ * given at creation: set_phase / resize_buffer / reset_prefill_buffer
+ * (GPU_Weight_Buffer.cpp:103-142, 310-379).  reset != 0 also drops residency and
+ * rewinds the cyclic queues (HtoD_Engine.cpp:284-311). */
+int moe_stage_set_active_slots(moe_stager* s, int32_t type, int32_t n_active, int32_t reset);
+/* Counters: copies issued, bytes issued. */
+int moe_stage_stats(moe_stager* s, int64_t* n_copies, int64_t* n_bytes);
+/* Host-blocking drain of the copy stream (teardown, tests). */
+int moe_stage_sync(moe_stager* s);
+int moe_stage_destroy(moe_stager* s);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOE_MI355_H */

@@ -1,0 +1,110 @@
+// Weighted combine for gfx950: inverse permutation, weighted sum over the k slots and
+// the shared-expert add in one pass over the expert outputs.
+//
+// Replaces the second half of moe_infer in the reference
+//   V3  modeling_deepseek_v3.py:702-710:  new_x[idxs] = outs;
+//        (new_x.view(n,k,h).float() * w[...,None]).sum(1).to(bf16)
+//   V2  modeling_deepseek_v2.py:744-757:  same with w cast to bf16 first (bf16 products)
+//   Mixtral (transformers 4.42.0): final.index_add_(0, top_x, expert_out * w) per expert
+// and `y = y + self.shared_experts(identity)` (modeling_deepseek_v3.py:624-625).
+// The reference materialises new_x [n,k,h] (and an fp32 copy of it); here each
+// output element is accumulated in a register from the k source rows.
+//
+// One block per token; a lane handles 8 consecutive bf16 (16 bytes) of the row, so
+// every global access is a full 16-byte vector and a wave covers 1 KiB contiguous.
+#include "common.h"
+
+namespace moe {
+namespace {
+
+constexpr int MAX_K = 16;
+
+template <int MODE>
+__global__ __launch_bounds__(256) void combine_kernel(const u32x4* __restrict__ y, const int32_t* __restrict__ pos,
+                                                      const int32_t* __restrict__ topk_idx,
+                                                      const float* __restrict__ topk_w, const u32x4* __restrict__ shared,
+                                                      int k, int chunks, u32x4* __restrict__ out) {
+    __shared__ int s_row[MAX_K];
+    __shared__ float s_w[MAX_K];
+    const int t = blockIdx.x;
+    if (threadIdx.x < k) {
+        // position of slot j in the summation order: the slot order itself, or (Mixtral, which
+        // adds expert by expert) the rank of its expert id among the k distinct ids of the token
+        const int j = threadIdx.x;
+        int a = j;
+        if (MODE == MOE_COMBINE_BF16_SEQ) {
+            const int ej = topk_idx[(size_t)t * k + j];
+            a = 0;
+            for (int i = 0; i < k; ++i) a += topk_idx[(size_t)t * k + i] < ej ? 1 : 0;
+        }
+        s_row[a] = pos[(size_t)t * k + j];
+        const float w = topk_w[(size_t)t * k + j];
+        s_w[a] = (MODE == MOE_COMBINE_F32) ? w : round_to_bf16(w);
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < chunks; c += 256) {
+        float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int a = 0; a < k; ++a) {
+            u32x4 v = y[(size_t)s_row[a] * chunks + c];
+            const float w = s_w[a];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float lo = __uint_as_float(v[i] << 16), hi = __uint_as_float(v[i] & 0xffff0000u);
+                if (MODE == MOE_COMBINE_F32) {
+                    acc[2 * i] = acc[2 * i] + lo * w;
+                    acc[2 * i + 1] = acc[2 * i + 1] + hi * w;
+                } else {
+                    acc[2 * i] = acc[2 * i] + round_to_bf16(lo * w);
+                    acc[2 * i + 1] = acc[2 * i + 1] + round_to_bf16(hi * w);
+                    if (MODE == MOE_COMBINE_BF16_SEQ) {
+                        acc[2 * i] = round_to_bf16(acc[2 * i]);
+                        acc[2 * i + 1] = round_to_bf16(acc[2 * i + 1]);
+                    }
+                }
+            }
+        }
+        u32x4 sh = {0, 0, 0, 0};
+        if (shared) sh = shared[(size_t)t * chunks + c];
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t lo = f32_to_bf16_bits(acc[2 * i]), hi = f32_to_bf16_bits(acc[2 * i + 1]);
+            if (shared) {  // bf16 + bf16 -> bf16, as torch adds two bf16 tensors
+                lo = f32_to_bf16_bits(bf16_bits_to_f32(lo) + __uint_as_float(sh[i] << 16));
+                hi = f32_to_bf16_bits(bf16_bits_to_f32(hi) + __uint_as_float(sh[i] & 0xffff0000u));
+            }
+            o[i] = lo | (hi << 16);
+        }
+        out[(size_t)t * chunks + c] = o;
+    }
+}
+
+}  // namespace
+}  // namespace moe
+
+extern "C" int moe_combine(const void* y, const int32_t* pos, const int32_t* topk_idx, const float* topk_w,
+                           const void* shared, int32_t n_tokens, int32_t top_k, int32_t hidden, int32_t mode,
+                           void* out, void* stream) {
+    using namespace moe;
+    MOE_REQUIRE(n_tokens >= 0, "moe_combine: n_tokens %d < 0", n_tokens);
+    if (n_tokens == 0) return MOE_OK;
+    MOE_REQUIRE(y && pos && topk_w && out, "moe_combine: NULL tensor pointer");
+    MOE_REQUIRE(top_k >= 1 && top_k <= MAX_K, "moe_combine: top_k %d outside [1,%d]", top_k, MAX_K);
+    MOE_REQUIRE(hidden > 0 && hidden % 8 == 0, "moe_combine: hidden %d must be a positive multiple of 8", hidden);
+    MOE_REQUIRE(mode >= MOE_COMBINE_F32 && mode <= MOE_COMBINE_BF16_SEQ, "moe_combine: bad mode %d", mode);
+    MOE_REQUIRE(mode != MOE_COMBINE_BF16_SEQ || topk_idx, "moe_combine: topk_idx is required for MOE_COMBINE_BF16_SEQ");
+    hipStream_t st = as_stream(stream);
+    dim3 grid(n_tokens), block(256);
+    const u32x4* yv = static_cast<const u32x4*>(y);
+    const u32x4* sv = static_cast<const u32x4*>(shared);
+    u32x4* ov = static_cast<u32x4*>(out);
+    const int chunks = hidden / 8;
+    if (mode == MOE_COMBINE_F32)
+        hipLaunchKernelGGL(combine_kernel<MOE_COMBINE_F32>, grid, block, 0, st, yv, pos, topk_idx, topk_w, sv, top_k, chunks, ov);
+    else if (mode == MOE_COMBINE_BF16_PROD)
+        hipLaunchKernelGGL(combine_kernel<MOE_COMBINE_BF16_PROD>, grid, block, 0, st, yv, pos, topk_idx, topk_w, sv, top_k, chunks, ov);
+    else
+        hipLaunchKernelGGL(combine_kernel<MOE_COMBINE_BF16_SEQ>, grid, block, 0, st, yv, pos, topk_idx, topk_w, sv, top_k, chunks, ov);
+    MOE_HIP_CHECK(hipGetLastError());
+    return MOE_OK;
+}

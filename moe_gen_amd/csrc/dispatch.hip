@@ -1,0 +1,206 @@
+// Token-to-expert dispatch for gfx950: per-expert histogram, exclusive prefix sum,
+// stable permutation and the row gather, all on the device (no host sync).
+//
+// Replaces the first half of moe_infer in the reference
+// (modeling_deepseek_v3.py:630-634 and :673, identical in modeling_deepseek_v2.py:672-676,715):
+//     cnts.scatter_(1, topk_ids, 1); tokens_per_expert = cnts.sum(0)
+//     idxs = topk_ids.view(-1).argsort();  sorted_tokens = x[idxs // k]
+// The sort is a stable counting sort: sorted row of flat entry i with expert e is
+//     offsets[e] + #{i' < i : idx[i'] == e}
+// which is a pure function of the index list, hence identical on every run.
+//
+// Three small kernels over the n*k index list (a few MB at most):
+//   1. block_histogram : each block counts its 2048-entry segment per expert (LDS atomics)
+//   2. scan_segments   : one wave per expert turns the per-segment counts into exclusive
+//                        bases across segments and writes counts[e]
+//   3. rank_scatter    : each block rebuilds offsets[] in LDS, ranks its entries with
+//                        wave-level match masks and writes perm / pos
+// and one bandwidth kernel:
+//   4. gather_rows     : xs[r] = x[perm[r] / k], one wave per row, 16 bytes per lane.
+#include "common.h"
+
+namespace moe {
+namespace {
+
+constexpr int SEG_PER_WAVE = 512;   // flat entries ranked by one wave
+constexpr int SEG_WAVES = 4;
+constexpr int SEG = SEG_PER_WAVE * SEG_WAVES;  // entries per block
+constexpr int MAX_E = 256;
+
+__global__ void zero_i32(int32_t* a, int na, int32_t* b, int nb) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < na) a[i] = 0;
+    if (i < nb) b[i] = 0;
+}
+
+__global__ __launch_bounds__(256) void block_histogram(const int32_t* __restrict__ idx, int64_t nk, int E,
+                                                       int32_t* __restrict__ seg_counts) {
+    __shared__ int hist[MAX_E];
+    for (int e = threadIdx.x; e < E; e += 256) hist[e] = 0;
+    __syncthreads();
+    const int64_t base = (int64_t)blockIdx.x * SEG;
+    for (int i = threadIdx.x; i < SEG; i += 256) {
+        int64_t g = base + i;
+        if (g < nk) {
+            int e = idx[g];
+            if ((unsigned)e < (unsigned)E) atomicAdd(&hist[e], 1);
+        }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += 256) seg_counts[(size_t)blockIdx.x * E + e] = hist[e];
+}
+
+// one wave per expert: in-place exclusive scan of seg_counts[:, e] over segments
+__global__ __launch_bounds__(256) void scan_segments(int32_t* __restrict__ seg_counts, int nseg, int E,
+                                                     int32_t* __restrict__ counts) {
+    const int lane = threadIdx.x & 63;
+    const int e = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (e >= E) return;
+    int carry = 0;
+    for (int b0 = 0; b0 < nseg; b0 += 64) {
+        int b = b0 + lane;
+        int v = b < nseg ? seg_counts[(size_t)b * E + e] : 0;
+        int inc = v;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            int o = __shfl_up(inc, d);
+            if (lane >= d) inc += o;
+        }
+        if (b < nseg) seg_counts[(size_t)b * E + e] = carry + inc - v;
+        carry += __shfl(inc, 63);
+    }
+    if (lane == 0) counts[e] = carry;
+}
+
+__global__ __launch_bounds__(256) void rank_scatter(const int32_t* __restrict__ idx, int64_t nk, int E,
+                                                    const int32_t* __restrict__ seg_base,
+                                                    const int32_t* __restrict__ counts,
+                                                    int32_t* __restrict__ offsets, int32_t* __restrict__ perm,
+                                                    int32_t* __restrict__ pos) {
+    __shared__ int off[MAX_E];                 // exclusive prefix sum of counts
+    __shared__ int whist[SEG_WAVES][MAX_E];    // per-wave counts, then per-wave running cursors
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    // offsets[e] = sum_{e' < e} counts[e'] : 256-wide scan by the whole block
+    int cv = tid < E ? counts[tid] : 0;
+    int inc = cv;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        int o = __shfl_up(inc, d);
+        if (lane >= d) inc += o;
+    }
+    __shared__ int wtot[4];
+    if (lane == 63) wtot[wave] = inc;
+    for (int e = tid; e < SEG_WAVES * MAX_E; e += 256) (&whist[0][0])[e] = 0;
+    __syncthreads();
+    int wpre = 0;
+    for (int w = 0; w < wave; ++w) wpre += wtot[w];
+    off[tid] = wpre + inc - cv;
+    if (blockIdx.x == 0) {
+        if (tid < E) offsets[tid] = wpre + inc - cv;
+        if (tid == E - 1) offsets[E] = wpre + inc;
+    }
+
+    // pass 1: counts of this wave's 512-entry slice
+    const int64_t wbase = (int64_t)blockIdx.x * SEG + (int64_t)wave * SEG_PER_WAVE;
+    for (int i = lane; i < SEG_PER_WAVE; i += 64) {
+        int64_t g = wbase + i;
+        if (g < nk) {
+            int e = idx[g];
+            if ((unsigned)e < (unsigned)E) atomicAdd(&whist[wave][e], 1);
+        }
+    }
+    __syncthreads();
+    // cursor of wave w for expert e = offsets[e] + base of this segment + counts of earlier waves
+    if (tid < E) {
+        int run = off[tid] + seg_base[(size_t)blockIdx.x * E + tid];
+#pragma unroll
+        for (int w = 0; w < SEG_WAVES; ++w) {
+            int c = whist[w][tid];
+            whist[w][tid] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+
+    // pass 2: stable rank inside the wave slice, 64 entries at a time in index order
+    int* cur = whist[wave];
+    for (int i0 = 0; i0 < SEG_PER_WAVE; i0 += 64) {
+        int64_t g = wbase + i0 + lane;
+        bool ok = g < nk;
+        int e = ok ? idx[g] : 0;
+        ok = ok && (unsigned)e < (unsigned)E;
+        uint64_t peers = __ballot(ok);
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            bool bit = (e >> b) & 1;
+            uint64_t bal = __ballot(bit);
+            peers &= bit ? bal : ~bal;
+        }
+        if (ok) {
+            uint64_t below = peers & ((1ull << lane) - 1ull);
+            int r = cur[e] + __popcll(below);
+            perm[r] = (int32_t)g;
+            pos[g] = r;
+        }
+        // every read of cur[] above precedes this update in the wave's LDS order
+        if (ok && (peers & ((1ull << lane) - 1ull)) == 0) cur[e] += __popcll(peers);
+    }
+}
+
+__global__ __launch_bounds__(256) void gather_rows(const u32x4* __restrict__ x, const int32_t* __restrict__ perm,
+                                                   int64_t nk, int k, int chunks, u32x4* __restrict__ xs) {
+    const int lane = threadIdx.x & 63;
+    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= nk) return;
+    const int t = perm[r] / k;
+    const u32x4* src = x + (size_t)t * chunks;
+    u32x4* dst = xs + (size_t)r * chunks;
+    for (int c = lane; c < chunks; c += 64) __builtin_nontemporal_store(src[c], dst + c);
+}
+
+}  // namespace
+}  // namespace moe
+
+extern "C" size_t moe_dispatch_workspace_bytes(int32_t n_tokens, int32_t top_k, int32_t n_experts) {
+    if (n_tokens <= 0 || top_k <= 0 || n_experts <= 0) return 256;
+    int64_t nk = (int64_t)n_tokens * top_k;
+    int64_t nseg = (nk + moe::SEG - 1) / moe::SEG;
+    return (size_t)(nseg * n_experts * 4 + 256);
+}
+
+extern "C" int moe_dispatch(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k, int32_t n_experts,
+                            int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* pos, const void* x,
+                            int32_t hidden, void* xs, void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace moe;
+    MOE_REQUIRE(n_tokens >= 0 && top_k >= 1, "moe_dispatch: bad n_tokens %d / top_k %d", n_tokens, top_k);
+    MOE_REQUIRE(n_experts >= 1 && n_experts <= MAX_E, "moe_dispatch: n_experts %d outside [1,%d]", n_experts, MAX_E);
+    MOE_REQUIRE(counts && offsets, "moe_dispatch: counts/offsets is NULL");
+    MOE_REQUIRE((x == nullptr) == (xs == nullptr), "moe_dispatch: x and xs must both be given or both be NULL");
+    const int64_t nk = (int64_t)n_tokens * top_k;
+    MOE_REQUIRE(nk < (int64_t)1 << 31, "moe_dispatch: n_tokens*top_k = %lld does not fit int32", (long long)nk);
+    hipStream_t st = as_stream(stream);
+    if (nk == 0) {
+        hipLaunchKernelGGL(zero_i32, dim3(2), dim3(256), 0, st, counts, n_experts, offsets, n_experts + 1);
+        MOE_HIP_CHECK(hipGetLastError());
+        return MOE_OK;
+    }
+    MOE_REQUIRE(topk_idx && perm && pos, "moe_dispatch: NULL index pointer");
+    if (x) MOE_REQUIRE(hidden > 0 && hidden % 8 == 0, "moe_dispatch: hidden %d must be a positive multiple of 8", hidden);
+    const int nseg = (int)((nk + SEG - 1) / SEG);
+    if (workspace == nullptr || workspace_bytes < (size_t)nseg * n_experts * 4) {
+        set_error("moe_dispatch: workspace %zu bytes, need %zu", workspace_bytes, (size_t)nseg * n_experts * 4);
+        return MOE_ERR_WORKSPACE;
+    }
+    int32_t* seg = static_cast<int32_t*>(workspace);
+    hipLaunchKernelGGL(block_histogram, dim3(nseg), dim3(256), 0, st, topk_idx, nk, n_experts, seg);
+    hipLaunchKernelGGL(scan_segments, dim3((n_experts + 3) / 4), dim3(256), 0, st, seg, nseg, n_experts, counts);
+    hipLaunchKernelGGL(rank_scatter, dim3(nseg), dim3(256), 0, st, topk_idx, nk, n_experts, seg, counts, offsets, perm,
+                       pos);
+    if (x) {
+        hipLaunchKernelGGL(gather_rows, dim3((unsigned)((nk + 3) / 4)), dim3(256), 0, st,
+                           static_cast<const u32x4*>(x), perm, nk, top_k, hidden / 8, static_cast<u32x4*>(xs));
+    }
+    MOE_HIP_CHECK(hipGetLastError());
+    return MOE_OK;
+}

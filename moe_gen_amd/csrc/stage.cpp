@@ -1,0 +1,287 @@
+// Expert-weight staging: a pool of HBM slots per module type, filled from pinned host
+// memory on a private copy stream in a fixed cyclic order, handed to the compute stream
+// by events.
+//
+// Replaces, for weights, the reference's copy worker and slot pool:
+//   HtoD_Engine::HtoD_Worker           core/HtoD_Engine/HtoD_Engine.cpp:201-268
+//   HtoD_Engine::blocking_copy_        core/HtoD_Engine/HtoD_Engine.cpp:112-118
+//   GPU_Weight_Buffer::acquireEmptyBuffer / releaseBuffer / get_weights /
+//     weights_copy_complete            core/GPU_Weight_Buffer/GPU_Weight_Buffer.cpp:146-259
+//   GPU_Weight_Buffer::resize_buffer / reset_prefill_buffer   :103-142, :310-379
+//   HtoD_Engine::reset_weight_copy_queue                      HtoD_Engine.cpp:284-311
+// The reference runs a host thread that copies one tensor at a time and synchronises
+// the stream after each, then wakes the consumer through a condition variable.  Here
+// no host thread exists and the host never waits: a copy is enqueued as soon as a slot
+// is free (pump), the consumer's stream waits on the copy's event (acquire), and the
+// next copy into a slot waits on the event recorded by the consumer when it let go of
+// the slot (release).  The copy order is the reference's: per type, the modules in the
+// order they were registered, cyclically, whether or not the router will use them.
+#include <cstring>
+#include <deque>
+#include <mutex>
+#include <vector>
+
+#include "common.h"
+
+namespace {
+
+struct Piece {
+    const void* src;
+    size_t bytes, dst_off;
+};
+
+struct Module {
+    int type = 0;
+    std::vector<Piece> pieces;
+    int slot = -1;               // -1: not resident
+    hipEvent_t ready = nullptr;  // copy finished (device backend)
+};
+
+struct Type {
+    size_t slot_bytes = 0;
+    int n_total = 0, n_active = 0;
+    uint8_t* mem = nullptr;
+    std::vector<int> owner;             // slot -> module id, -1 free
+    std::vector<hipEvent_t> freed;      // recorded on the consumer stream at release
+    std::vector<char> freed_valid;
+    std::vector<int> order;             // registration order
+    std::deque<int> fifo;               // cyclic copy queue
+};
+
+}  // namespace
+
+struct moe_stager {
+    int backend = MOE_STAGE_DEVICE;
+    hipStream_t copy_stream = nullptr;
+    std::vector<Type> types;
+    std::vector<Module> modules;
+    int64_t n_copies = 0, n_bytes = 0;
+    std::mutex mu;
+};
+
+namespace {
+
+int find_free(const Type& t) {
+    for (int s = 0; s < t.n_active; ++s)
+        if (t.owner[s] < 0) return s;
+    return -1;
+}
+
+// one turn of the copy worker for one type; returns 1 if a copy was enqueued, 0 if not, <0 on error
+int pump_type(moe_stager* st, int ti) {
+    Type& t = st->types[ti];
+    if (t.fifo.empty()) return 0;
+    const int slot = find_free(t);
+    if (slot < 0) return 0;
+    const int id = t.fifo.front();
+    Module& m = st->modules[id];
+    if (m.slot >= 0) return 0;  // next in line still occupies a slot: nothing to do until it is released
+    t.fifo.pop_front();
+    uint8_t* dst = t.mem + (size_t)slot * t.slot_bytes;
+    if (st->backend == MOE_STAGE_DEVICE) {
+        if (t.freed_valid[slot]) {
+            MOE_HIP_CHECK(hipStreamWaitEvent(st->copy_stream, t.freed[slot], 0));
+            t.freed_valid[slot] = 0;
+        }
+        for (const Piece& p : m.pieces)
+            MOE_HIP_CHECK(hipMemcpyAsync(dst + p.dst_off, p.src, p.bytes, hipMemcpyHostToDevice, st->copy_stream));
+        MOE_HIP_CHECK(hipEventRecord(m.ready, st->copy_stream));
+    } else {
+        for (const Piece& p : m.pieces) std::memcpy(dst + p.dst_off, p.src, p.bytes);
+    }
+    for (const Piece& p : m.pieces) st->n_bytes += (int64_t)p.bytes;
+    st->n_copies += 1;
+    t.owner[slot] = id;
+    m.slot = slot;
+    t.fifo.push_back(id);  // the reference pushes the name back for the next pass
+    return 1;
+}
+
+int pump_all(moe_stager* st) {
+    int n = 0;
+    for (size_t ti = 0; ti < st->types.size(); ++ti) {
+        for (;;) {
+            int r = pump_type(st, (int)ti);
+            if (r < 0) return r;
+            if (r == 0) break;
+            ++n;
+        }
+    }
+    return n;
+}
+
+}  // namespace
+
+extern "C" int moe_stage_create(moe_stager** out, int32_t n_types, const size_t* slot_bytes, const int32_t* n_slots,
+                                void* const* slot_mem, int32_t backend) {
+    MOE_REQUIRE(out && slot_bytes && n_slots && slot_mem, "moe_stage_create: NULL argument");
+    MOE_REQUIRE(n_types >= 1 && n_types <= 64, "moe_stage_create: n_types %d outside [1,64]", n_types);
+    MOE_REQUIRE(backend == MOE_STAGE_DEVICE || backend == MOE_STAGE_HOST_MEMCPY, "moe_stage_create: bad backend %d",
+                backend);
+    moe_stager* st = new moe_stager();
+    st->backend = backend;
+    st->types.resize(n_types);
+    for (int i = 0; i < n_types; ++i) {
+        Type& t = st->types[i];
+        if (n_slots[i] < 1 || slot_bytes[i] == 0 || slot_mem[i] == nullptr) {
+            moe::set_error("moe_stage_create: type %d needs >= 1 slot, non-zero slot size and slot memory", i);
+            delete st;
+            return MOE_ERR_INVALID;
+        }
+        t.slot_bytes = slot_bytes[i];
+        t.n_total = t.n_active = n_slots[i];
+        t.mem = static_cast<uint8_t*>(slot_mem[i]);
+        t.owner.assign(t.n_total, -1);
+        t.freed.assign(t.n_total, nullptr);
+        t.freed_valid.assign(t.n_total, 0);
+    }
+    if (backend == MOE_STAGE_DEVICE) {
+        hipError_t e = hipStreamCreateWithFlags(&st->copy_stream, hipStreamNonBlocking);
+        if (e != hipSuccess) {
+            moe::set_error("moe_stage_create: hipStreamCreateWithFlags: %s", hipGetErrorString(e));
+            delete st;
+            return MOE_ERR_HIP;
+        }
+        for (Type& t : st->types)
+            for (int s = 0; s < t.n_total; ++s) {
+                e = hipEventCreateWithFlags(&t.freed[s], hipEventDisableTiming);
+                if (e != hipSuccess) {
+                    moe::set_error("moe_stage_create: hipEventCreateWithFlags: %s", hipGetErrorString(e));
+                    return MOE_ERR_HIP;
+                }
+            }
+    }
+    *out = st;
+    return MOE_OK;
+}
+
+extern "C" int moe_stage_add_module(moe_stager* st, int32_t type, int32_t n_tensors, const void* const* src,
+                                    const size_t* bytes, const size_t* dst_offsets) {
+    MOE_REQUIRE(st && src && bytes && dst_offsets, "moe_stage_add_module: NULL argument");
+    std::lock_guard<std::mutex> lk(st->mu);
+    MOE_REQUIRE(type >= 0 && type < (int)st->types.size(), "moe_stage_add_module: bad type %d", type);
+    MOE_REQUIRE(n_tensors >= 1, "moe_stage_add_module: n_tensors %d < 1", n_tensors);
+    Type& t = st->types[type];
+    Module m;
+    m.type = type;
+    for (int i = 0; i < n_tensors; ++i) {
+        MOE_REQUIRE(src[i] != nullptr, "moe_stage_add_module: tensor %d has a NULL source", i);
+        MOE_REQUIRE(dst_offsets[i] + bytes[i] <= t.slot_bytes,
+                    "moe_stage_add_module: tensor %d (%zu bytes at offset %zu) overruns the %zu-byte slot", i, bytes[i],
+                    dst_offsets[i], t.slot_bytes);
+        m.pieces.push_back(Piece{src[i], bytes[i], dst_offsets[i]});
+    }
+    if (st->backend == MOE_STAGE_DEVICE) MOE_HIP_CHECK(hipEventCreateWithFlags(&m.ready, hipEventDisableTiming));
+    const int id = (int)st->modules.size();
+    st->modules.push_back(std::move(m));
+    t.order.push_back(id);
+    t.fifo.push_back(id);
+    return id;
+}
+
+extern "C" int moe_stage_pump(moe_stager* st) {
+    MOE_REQUIRE(st, "moe_stage_pump: NULL stager");
+    std::lock_guard<std::mutex> lk(st->mu);
+    return pump_all(st);
+}
+
+extern "C" int moe_stage_acquire(moe_stager* st, int32_t id, void* stream, int32_t* slot) {
+    MOE_REQUIRE(st && slot, "moe_stage_acquire: NULL argument");
+    std::lock_guard<std::mutex> lk(st->mu);
+    MOE_REQUIRE(id >= 0 && id < (int)st->modules.size(), "moe_stage_acquire: unknown module id %d", id);
+    Module& m = st->modules[id];
+    while (m.slot < 0) {
+        int r = pump_all(st);
+        if (r < 0) return r;
+        if (r == 0 && m.slot < 0) {
+            moe::set_error("moe_stage_acquire: module %d cannot be scheduled: every slot of type %d is held "
+                           "(release or clear earlier modules first)", id, m.type);
+            return MOE_ERR_STATE;
+        }
+    }
+    if (st->backend == MOE_STAGE_DEVICE) MOE_HIP_CHECK(hipStreamWaitEvent(moe::as_stream(stream), m.ready, 0));
+    *slot = m.slot;
+    return MOE_OK;
+}
+
+extern "C" int moe_stage_release(moe_stager* st, int32_t id, void* stream) {
+    MOE_REQUIRE(st, "moe_stage_release: NULL stager");
+    std::lock_guard<std::mutex> lk(st->mu);
+    MOE_REQUIRE(id >= 0 && id < (int)st->modules.size(), "moe_stage_release: unknown module id %d", id);
+    Module& m = st->modules[id];
+    if (m.slot < 0) {
+        moe::set_error("moe_stage_release: module %d is not resident", id);
+        return MOE_ERR_STATE;
+    }
+    Type& t = st->types[m.type];
+    if (st->backend == MOE_STAGE_DEVICE) {
+        MOE_HIP_CHECK(hipEventRecord(t.freed[m.slot], moe::as_stream(stream)));
+        t.freed_valid[m.slot] = 1;
+    }
+    t.owner[m.slot] = -1;
+    m.slot = -1;
+    int r = pump_all(st);  // the worker refills a freed slot at once
+    return r < 0 ? r : MOE_OK;
+}
+
+extern "C" int moe_stage_resident(moe_stager* st, int32_t id) {
+    MOE_REQUIRE(st, "moe_stage_resident: NULL stager");
+    std::lock_guard<std::mutex> lk(st->mu);
+    MOE_REQUIRE(id >= 0 && id < (int)st->modules.size(), "moe_stage_resident: unknown module id %d", id);
+    return st->modules[id].slot >= 0 ? 1 : 0;
+}
+
+extern "C" int moe_stage_set_active_slots(moe_stager* st, int32_t type, int32_t n_active, int32_t reset) {
+    MOE_REQUIRE(st, "moe_stage_set_active_slots: NULL stager");
+    std::lock_guard<std::mutex> lk(st->mu);
+    MOE_REQUIRE(type >= 0 && type < (int)st->types.size(), "moe_stage_set_active_slots: bad type %d", type);
+    Type& t = st->types[type];
+    MOE_REQUIRE(n_active >= 1 && n_active <= t.n_total, "moe_stage_set_active_slots: %d outside [1,%d]", n_active,
+                t.n_total);
+    if (reset) {
+        if (st->backend == MOE_STAGE_DEVICE) MOE_HIP_CHECK(hipStreamSynchronize(st->copy_stream));
+        for (int s = 0; s < t.n_total; ++s) {
+            if (t.owner[s] >= 0) st->modules[t.owner[s]].slot = -1;
+            t.owner[s] = -1;
+        }
+        t.fifo.assign(t.order.begin(), t.order.end());
+    } else {
+        for (int s = n_active; s < t.n_total; ++s)
+            if (t.owner[s] >= 0) {
+                moe::set_error("moe_stage_set_active_slots: slot %d of type %d is still occupied", s, type);
+                return MOE_ERR_STATE;
+            }
+    }
+    t.n_active = n_active;
+    return MOE_OK;
+}
+
+extern "C" int moe_stage_stats(moe_stager* st, int64_t* n_copies, int64_t* n_bytes) {
+    MOE_REQUIRE(st, "moe_stage_stats: NULL stager");
+    std::lock_guard<std::mutex> lk(st->mu);
+    if (n_copies) *n_copies = st->n_copies;
+    if (n_bytes) *n_bytes = st->n_bytes;
+    return MOE_OK;
+}
+
+extern "C" int moe_stage_sync(moe_stager* st) {
+    MOE_REQUIRE(st, "moe_stage_sync: NULL stager");
+    std::lock_guard<std::mutex> lk(st->mu);
+    if (st->backend == MOE_STAGE_DEVICE) MOE_HIP_CHECK(hipStreamSynchronize(st->copy_stream));
+    return MOE_OK;
+}
+
+extern "C" int moe_stage_destroy(moe_stager* st) {
+    if (!st) return MOE_OK;
+    if (st->backend == MOE_STAGE_DEVICE) {
+        (void)hipStreamSynchronize(st->copy_stream);
+        for (Module& m : st->modules)
+            if (m.ready) (void)hipEventDestroy(m.ready);
+        for (Type& t : st->types)
+            for (hipEvent_t ev : t.freed)
+                if (ev) (void)hipEventDestroy(ev);
+        (void)hipStreamDestroy(st->copy_stream);
+    }
+    delete st;
+    return MOE_OK;
+}

@@ -1,0 +1,98 @@
+"""DeepSeek-V2 MoE layer with the reference's module surface
+(modeling_deepseek_v2.py:425-758): DeepseekV2MLP, MoEGate, DeepseekV2MoE."""
+from __future__ import annotations
+
+import math
+
+import torch
+from torch import nn
+
+from . import ops
+from .block import SwiGLUMLP, _require_silu, moe_forward
+
+
+class DeepseekV2MLP(SwiGLUMLP):
+    """modeling_deepseek_v2.py:425-453."""
+
+    def __init__(self, config, hidden_size=None, intermediate_size=None):
+        _require_silu(config)
+        super().__init__(config.hidden_size if hidden_size is None else hidden_size,
+                         config.intermediate_size if intermediate_size is None else intermediate_size)
+        self.config = config
+
+
+def _spec(gate) -> ops.RouterSpec:
+    if gate.scoring_func != "softmax":
+        raise NotImplementedError(f"insupportable scoring function for MoE gating: {gate.scoring_func}")
+    if gate.topk_method not in ("greedy", "group_limited_greedy"):
+        raise NotImplementedError(f"insupportable TopK function for MoE gating: {gate.topk_method}")
+    grouped = gate.topk_method == "group_limited_greedy"
+    return ops.RouterSpec(gate.n_routed_experts, gate.top_k, "softmax", gate.topk_method,
+                          gate.n_group if grouped else 1, gate.topk_group if grouped else 1,
+                          bool(gate.norm_topk_prob), 1, float(gate.routed_scaling_factor), 1e-20)
+
+
+class MoEGate(nn.Module):
+    """modeling_deepseek_v2.py:456-566: softmax scores, greedy or group-limited greedy top-k
+    (group score = its best expert); renormalise OR scale (:529-533).  Inference only: the
+    auxiliary loss (:535-565) is a training quantity and is returned as None."""
+
+    def __init__(self, config):
+        super().__init__()
+        self.config = config
+        self.top_k = config.num_experts_per_tok
+        self.n_routed_experts = config.n_routed_experts
+        self.routed_scaling_factor = config.routed_scaling_factor
+        self.scoring_func = config.scoring_func
+        self.alpha = getattr(config, "aux_loss_alpha", 0.0)
+        self.seq_aux = getattr(config, "seq_aux", True)
+        self.topk_method = config.topk_method
+        self.n_group = config.n_group
+        self.topk_group = config.topk_group
+        self.norm_topk_prob = config.norm_topk_prob
+        self.gating_dim = config.hidden_size
+        self.weight = nn.Parameter(torch.empty((self.n_routed_experts, self.gating_dim)))
+        self.reset_parameters()
+
+    def reset_parameters(self) -> None:
+        nn.init.kaiming_uniform_(self.weight, a=math.sqrt(5))
+
+    @torch.no_grad()
+    def forward(self, hidden_states):
+        """-> (topk_idx int64 [n,k], topk_weight fp32 [n,k], aux_loss=None)."""
+        if self.training:
+            raise NotImplementedError("inference only: the auxiliary loss is not computed")
+        from .block import _gate_weight_bf16
+        h = hidden_states.shape[-1]
+        x = hidden_states.reshape(-1, h)
+        cache = self.__dict__.setdefault("_moe_cache", {})
+        idx, w, _ = ops.router(x.contiguous(), _gate_weight_bf16(self.weight, cache), None, _spec(self))
+        return idx.to(torch.int64), w, None
+
+
+class DeepseekV2MoE(nn.Module):
+    """modeling_deepseek_v2.py:592-758, inference path (the training branch :648-661 is not built)."""
+
+    def __init__(self, config):
+        super().__init__()
+        self.config = config
+        self.num_experts_per_tok = config.num_experts_per_tok
+        if getattr(config, "ep_size", 1) > 1:
+            raise NotImplementedError("expert parallelism (ep_size > 1) is outside this single-GPU build")
+        self.ep_size, self.experts_per_rank, self.ep_rank = 1, config.n_routed_experts, 0
+        self.experts = nn.ModuleList(
+            [DeepseekV2MLP(config, intermediate_size=config.moe_intermediate_size)
+             for _ in range(config.n_routed_experts)])
+        self.gate = MoEGate(config)
+        if config.n_shared_experts is not None:
+            self.shared_experts = DeepseekV2MLP(
+                config=config, intermediate_size=config.moe_intermediate_size * config.n_shared_experts)
+
+    @torch.no_grad()
+    def forward(self, hidden_states):
+        if self.training:
+            raise NotImplementedError("inference only (the reference's moe_infer path)")
+        shared = self.shared_experts if self.config.n_shared_experts is not None else None
+        out, _ = moe_forward(self, hidden_states, _spec(self.gate), self.gate.weight, None, self.experts, shared,
+                             ops.COMBINE_BF16_PROD)
+        return out

@@ -1,0 +1,182 @@
+"""Expert-weight staging with the three verbs MoE-Gen's engine exposes to the model code
+(core/MoE_Gen_Binding.cpp:45-65): get_weights, free_weights_buffer, clear_expert_buffer, plus
+set_phase.  The slot pool and the copy queue live in libmoe_mi355.so (moe_stage_*); this class
+maps module keys ("routed_expert_{L}_{e}", "shared_expert_{L}", Wrapper.py:457-468) to ids and
+wraps slot memory as torch tensors."""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import _native as N
+
+_ALIGN = 256
+
+
+def _nbytes(shape, dtype) -> int:
+    n = 1
+    for s in shape:
+        n *= int(s)
+    return n * torch.empty((), dtype=dtype).element_size()
+
+
+class Stager:
+    """module_shapes: {module_type: {tensor_name: (shape, dtype)}} -- the reference's
+    GPU_Buffer_Config.module_shapes (deepseekv3_initializer.py:938-957);
+    n_slots: {module_type: slots in the prefill phase}; n_slots_decoding: optional larger
+    counts for the decoding phase (num_decoding_module_buffer, :918-927);
+    backend "device": slots in HBM, sources must be pinned host tensors;
+    backend "host": slots in host memory, plain memcpy (host-only tests)."""
+
+    def __init__(self, module_shapes: dict, n_slots: dict, device="cuda", n_slots_decoding: dict | None = None,
+                 model_type: str = "", num_hidden_layers: int = 0, num_local_experts: int = 0,
+                 backend: str = "device"):
+        self.backend = backend
+        self.device = torch.device("cpu") if backend == "host" else torch.device(device)
+        self.model_type = model_type
+        self.num_hidden_layers = num_hidden_layers
+        self.num_local_experts = num_local_experts
+        self.types = list(module_shapes.keys())
+        self.layout = {}       # type -> {name: (offset, bytes, shape, dtype)}
+        self.pools = {}        # type -> uint8 tensor [n_total, slot_bytes]
+        self.n_prefill = dict(n_slots)
+        self.n_decoding = dict(n_slots_decoding or n_slots)
+        slot_bytes, totals, mems = [], [], []
+        for t in self.types:
+            off, lay = 0, {}
+            for name, (shape, dtype) in module_shapes[t].items():
+                b = _nbytes(shape, dtype)
+                lay[name] = (off, b, tuple(shape), dtype)
+                off += -(-b // _ALIGN) * _ALIGN
+            self.layout[t] = lay
+            total = max(self.n_prefill[t], self.n_decoding.get(t, 0))
+            self.pools[t] = torch.zeros((total, off), dtype=torch.uint8, device=self.device)
+            slot_bytes.append(off)
+            totals.append(total)
+            mems.append(self.pools[t].data_ptr())
+        nt = len(self.types)
+        self._h = ctypes.c_void_p()
+        N.check(N.lib().moe_stage_create(ctypes.byref(self._h), nt, (ctypes.c_size_t * nt)(*slot_bytes),
+                                         (ctypes.c_int32 * nt)(*totals), (ctypes.c_void_p * nt)(*mems),
+                                         1 if backend == "host" else 0), "moe_stage_create")
+        for i, t in enumerate(self.types):
+            if self.n_prefill[t] != totals[i]:
+                N.check(N.lib().moe_stage_set_active_slots(self._h, i, self.n_prefill[t], 0),
+                        "moe_stage_set_active_slots")
+        self.ids = {}          # module_key -> id
+        self.type_of = {}      # module_key -> type
+        self._src = []         # keeps the host tensors alive
+        self.phase = "prefill"
+
+    def _stream(self):
+        return None if self.backend == "host" else torch.cuda.current_stream().cuda_stream
+
+    def add_module(self, module_key: str, module_type: str, tensors: dict) -> int:
+        """Register one module (Weights_Storage's module_key -> tensor_key -> host buffer map,
+        core/Weights_Storage/Weights_Storage.cpp:52-90) at the tail of its type's copy queue."""
+        lay = self.layout[module_type]
+        if set(tensors) != set(lay):
+            raise RuntimeError(f"module {module_key}: tensors {sorted(tensors)} do not match the slot layout {sorted(lay)}")
+        n = len(lay)
+        src, nbytes, offs = [], [], []
+        for name, (off, b, shape, dtype) in lay.items():
+            t = tensors[name]
+            if tuple(t.shape) != shape or t.dtype != dtype or not t.is_contiguous() or t.is_cuda:
+                raise RuntimeError(f"module {module_key}.{name}: expected a contiguous host {dtype} tensor of shape {shape}")
+            if self.backend == "device" and not t.is_pinned():
+                raise RuntimeError(f"module {module_key}.{name}: host tensor must be pinned (allocate with pin_memory=True)")
+            src.append(t.data_ptr()); nbytes.append(b); offs.append(off)
+            self._src.append(t)
+        mid = N.lib().moe_stage_add_module(self._h, self.types.index(module_type), n, (ctypes.c_void_p * n)(*src),
+                                           (ctypes.c_size_t * n)(*nbytes), (ctypes.c_size_t * n)(*offs))
+        if mid < 0:
+            N.check(mid, "moe_stage_add_module")
+        self.ids[module_key] = mid
+        self.type_of[module_key] = module_type
+        return mid
+
+    def pump(self) -> int:
+        r = N.lib().moe_stage_pump(self._h)
+        if r < 0:
+            N.check(r, "moe_stage_pump")
+        return r
+
+    def _id(self, module_key: str) -> int:
+        if module_key not in self.ids:
+            # the reference throws from Weights_Storage::get_module_weights_storage (:82-87)
+            raise RuntimeError(f"Module key not found: {module_key}")
+        return self.ids[module_key]
+
+    def get_weights(self, module_key: str) -> dict:
+        """Tensors aliasing the slot that holds `module_key`; the current stream is made to wait
+        for the copy (GPU_Weight_Buffer::get_weights, GPU_Weight_Buffer.cpp:171-246, without the
+        host-side wait)."""
+        slot = ctypes.c_int32(-1)
+        N.check(N.lib().moe_stage_acquire(self._h, self._id(module_key), self._stream(), ctypes.byref(slot)),
+                "moe_stage_acquire")
+        t = self.type_of[module_key]
+        row = self.pools[t][slot.value]
+        return {name: row[off:off + b].view(dtype).view(shape) for name, (off, b, shape, dtype) in self.layout[t].items()}
+
+    def free_weights_buffer(self, module_key: str) -> None:
+        N.check(N.lib().moe_stage_release(self._h, self._id(module_key), self._stream()), "moe_stage_release")
+
+    def resident(self, module_key: str) -> bool:
+        r = N.lib().moe_stage_resident(self._h, self._id(module_key))
+        if r < 0:
+            N.check(r, "moe_stage_resident")
+        return bool(r)
+
+    def _prev_layer(self, layer_idx: int) -> int:
+        # GPU_Weight_Buffer.cpp:279-294: the first MoE layers wrap to the last layer
+        if self.model_type == "deepseek_v2" and layer_idx in (0, 1):
+            return self.num_hidden_layers - 1
+        if self.model_type == "deepseek_v3" and 0 <= layer_idx <= 3:
+            return self.num_hidden_layers - 1
+        return layer_idx - 1
+
+    def clear_expert_buffer(self, layer_idx: int, expert_idx: int) -> None:
+        """Release slots still held by routed experts that were prefetched but skipped (no tokens):
+        experts < expert_idx of this layer and every expert of the previous MoE layer
+        (GPU_Weight_Buffer::clear_expert_buffer, GPU_Weight_Buffer.cpp:261-308)."""
+        keys = [f"routed_expert_{layer_idx}_{e}" for e in range(expert_idx)]
+        pl = self._prev_layer(layer_idx)
+        keys += [f"routed_expert_{pl}_{e}" for e in range(self.num_local_experts)]
+        for key in keys:
+            if key in self.ids and self.resident(key):
+                self.free_weights_buffer(key)
+
+    def set_phase(self, phase: str) -> None:
+        """"decoding" grows the routed-expert pool (resize_buffer, GPU_Weight_Buffer.cpp:103-142);
+        "prefill" shrinks it back, drops residency and rewinds the queues
+        (reset_prefill_buffer :310-379, reset_weight_copy_queue HtoD_Engine.cpp:284-311)."""
+        if phase not in ("prefill", "decoding"):
+            raise RuntimeError(f"unknown phase {phase!r}")
+        for i, t in enumerate(self.types):
+            if phase == "decoding":
+                N.check(N.lib().moe_stage_set_active_slots(self._h, i, self.n_decoding.get(t, self.n_prefill[t]), 0),
+                        "moe_stage_set_active_slots")
+            else:
+                N.check(N.lib().moe_stage_set_active_slots(self._h, i, self.n_prefill[t], 1),
+                        "moe_stage_set_active_slots")
+        self.phase = phase
+
+    def stats(self):
+        c, b = ctypes.c_int64(), ctypes.c_int64()
+        N.check(N.lib().moe_stage_stats(self._h, ctypes.byref(c), ctypes.byref(b)), "moe_stage_stats")
+        return c.value, b.value
+
+    def sync(self) -> None:
+        N.check(N.lib().moe_stage_sync(self._h), "moe_stage_sync")
+
+    def close(self) -> None:
+        if getattr(self, "_h", None) is not None and self._h.value:
+            N.lib().moe_stage_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
