@@ -123,15 +123,18 @@ int moe_dispatch(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k, int32
  *   act       device bf16 [n_rows, I]  scratch for a
  *   y         device bf16 [n_rows, h]  out
  *   workspace device, at least moe_grouped_workspace_bytes(n_rows, E) bytes
+ *   phases    MOE_PHASE_GATE_UP (writes act), MOE_PHASE_DOWN (reads act, writes y) or
+ *             MOE_PHASE_BOTH; the two launches can be issued (and timed) separately
  * Requires h % 64 == 0 and I % 64 == 0.
  */
+enum { MOE_PHASE_GATE_UP = 1, MOE_PHASE_DOWN = 2, MOE_PHASE_BOTH = 3 };
 size_t moe_grouped_workspace_bytes(int32_t n_rows, int32_t n_experts);
 int moe_grouped_swiglu_bf16(const void* x, const int32_t* row_map,
                             const void* const* w_gate, const void* const* w_up,
                             const void* const* w_down, const int32_t* offsets,
                             int32_t n_rows, int32_t n_experts, int32_t hidden, int32_t inter,
-                            void* act, void* y, void* workspace, size_t workspace_bytes,
-                            void* stream);
+                            void* act, void* y, int32_t phases, void* workspace,
+                            size_t workspace_bytes, void* stream);
 
 /*
  * W8A16 variant: weights are fp8 e4m3fn with one fp32 scale per 128x128 block;
@@ -147,8 +150,8 @@ int moe_grouped_swiglu_w8a16(const void* x, const int32_t* row_map,
                              const float* const* s_gate, const float* const* s_up,
                              const float* const* s_down, const int32_t* offsets,
                              int32_t n_rows, int32_t n_experts, int32_t hidden, int32_t inter,
-                             void* act, void* y, void* workspace, size_t workspace_bytes,
-                             void* stream);
+                             void* act, void* y, int32_t phases, void* workspace,
+                             size_t workspace_bytes, void* stream);
 
 /*
  * Stand-alone block dequantisation (Wrapper.py:109-138), used by tests and by

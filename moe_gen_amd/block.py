@@ -11,6 +11,62 @@ from . import ops
 FP8 = torch.float8_e4m3fn
 
 
+class StageTimer:
+    """Optional per-stage timing of a block's forward with events recorded on the stream the
+    kernels are launched on (torch's current stream).  Attach as `block.stage_timer`."""
+
+    def __init__(self):
+        self.spans = []      # (name, start_event, end_event)
+
+    class _Span:
+        def __init__(self, timer, name):
+            self.t, self.name = timer, name
+
+        def __enter__(self):
+            self.a = torch.cuda.Event(enable_timing=True)
+            self.a.record()
+
+        def __exit__(self, *exc):
+            b = torch.cuda.Event(enable_timing=True)
+            b.record()
+            self.t.spans.append((self.name, self.a, b))
+
+    def span(self, name):
+        return StageTimer._Span(self, name)
+
+    def totals_ms(self) -> dict:
+        """name -> list of durations (ms); call after torch.cuda.synchronize()."""
+        out = {}
+        for name, a, b in self.spans:
+            out.setdefault(name, []).append(a.elapsed_time(b))
+        return out
+
+
+class _NoSpan:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+def _span(timer, name):
+    return timer.span(name) if timer is not None else _NoSpan()
+
+
+def _grouped(timer, tag, x, row_map, ptrs, offsets, n_rows):
+    """Both launches of the expert MLP; split (and timed per launch) when a timer is attached."""
+    if timer is None:
+        return ops.grouped_swiglu(x, row_map, ptrs, offsets, n_rows)
+    act = torch.empty((n_rows, ptrs.inter), dtype=torch.bfloat16, device=x.device)
+    y = torch.empty((n_rows, ptrs.hidden), dtype=torch.bfloat16, device=x.device)
+    with timer.span(tag + "_gate_up"):
+        ops.grouped_swiglu(x, row_map, ptrs, offsets, n_rows, act, y, ops.PHASE_GATE_UP)
+    with timer.span(tag + "_down"):
+        ops.grouped_swiglu(x, row_map, ptrs, offsets, n_rows, act, y, ops.PHASE_DOWN)
+    return y
+
+
 def _require_silu(config):
     act = getattr(config, "hidden_act", "silu")
     if act != "silu":
@@ -156,17 +212,17 @@ def moe_forward(block, hidden_states: torch.Tensor, spec: ops.RouterSpec, gate_w
     cache = block.__dict__.setdefault("_moe_cache", {})
     gw = _gate_weight_bf16(gate_weight, cache)
     b = None if bias is None else bias.data.to(torch.float32)
-    idx, w, logits = ops.router(x, gw, b, spec, want_logits)
+    timer = getattr(block, "stage_timer", None)
+    with _span(timer, "router"):
+        idx, w, logits = ops.router(x, gw, b, spec, want_logits)
     block.last_topk_idx, block.last_topk_weight = idx, w
     fused_gather = getattr(block, "fused_gather", True)
-    counts, offsets, perm, pos, xs = ops.dispatch(idx, E, None if fused_gather else x)
+    with _span(timer, "dispatch"):
+        counts, offsets, perm, pos, xs = ops.dispatch(idx, E, None if fused_gather else x)
+        row_map = torch.div(perm, k, rounding_mode="floor").to(torch.int32) if fused_gather else None
     block.last_counts = counts
     ptrs, keys = collect_pointers(list(experts), cache.setdefault("routed", {}))
-    if fused_gather:
-        row_map = torch.div(perm, k, rounding_mode="floor").to(torch.int32)
-        y = ops.grouped_swiglu(x, row_map, ptrs, offsets, n * k)
-    else:
-        y = ops.grouped_swiglu(xs, None, ptrs, offsets, n * k)
+    y = _grouped(timer, "routed", x if fused_gather else xs, row_map, ptrs, offsets, n * k)
     for eng, key in keys:
         eng.free_weights_buffer(key)
     sh = None
@@ -176,8 +232,9 @@ def moe_forward(block, hidden_states: torch.Tensor, spec: ops.RouterSpec, gate_w
         if so is None or so[0] != n or so[1].device != x.device:
             so = (n, torch.tensor([0, n], dtype=torch.int32, device=x.device))
             cache["shared_off"] = so
-        sh = ops.grouped_swiglu(x, None, sp, so[1], n)
+        sh = _grouped(timer, "shared", x, None, sp, so[1], n)
         for eng, key in skeys:
             eng.free_weights_buffer(key)
-    out = ops.combine(y, pos, idx, w, sh, combine_mode)
+    with _span(timer, "combine"):
+        out = ops.combine(y, pos, idx, w, sh, combine_mode)
     return out.view(*shape), logits

@@ -343,8 +343,9 @@ template <bool W8>
 int grouped_swiglu(const void* x, const int32_t* row_map, const void* const* w_gate, const void* const* w_up,
                    const void* const* w_down, const float* const* s_gate, const float* const* s_up,
                    const float* const* s_down, const int32_t* offsets, int32_t n_rows, int32_t n_experts,
-                   int32_t hidden, int32_t inter, void* act, void* y, void* stream, const char* who) {
+                   int32_t hidden, int32_t inter, void* act, void* y, int32_t phases, void* stream, const char* who) {
     MOE_REQUIRE(n_rows >= 0, "%s: n_rows %d < 0", who, n_rows);
+    MOE_REQUIRE(phases >= MOE_PHASE_GATE_UP && phases <= MOE_PHASE_BOTH, "%s: bad phases %d", who, phases);
     if (n_rows == 0) return MOE_OK;
     MOE_REQUIRE(x && w_gate && w_up && w_down && offsets && act && y, "%s: NULL pointer argument", who);
     MOE_REQUIRE(!W8 || (s_gate && s_up && s_down), "%s: NULL scale pointer array", who);
@@ -362,8 +363,11 @@ int grouped_swiglu(const void* x, const int32_t* row_map, const void* const* w_g
     g1.c = static_cast<uint16_t*>(act);
     g1.E = n_experts; g1.K = hidden; g1.N = inter;
     g1.n_tiles_n = (inter + 127) / 128;
-    int rc = launch_mt<true, W8>(g1, n_rows, st);
-    if (rc != MOE_OK) return rc;
+    if (phases & MOE_PHASE_GATE_UP) {
+        int rc = launch_mt<true, W8>(g1, n_rows, st);
+        if (rc != MOE_OK) return rc;
+    }
+    if (!(phases & MOE_PHASE_DOWN)) return MOE_OK;
     GemmArgs g2{};
     g2.a = static_cast<const uint16_t*>(act);
     g2.row_map = nullptr;
@@ -406,19 +410,19 @@ extern "C" size_t moe_grouped_workspace_bytes(int32_t, int32_t) { return 256; }
 extern "C" int moe_grouped_swiglu_bf16(const void* x, const int32_t* row_map, const void* const* w_gate,
                                        const void* const* w_up, const void* const* w_down, const int32_t* offsets,
                                        int32_t n_rows, int32_t n_experts, int32_t hidden, int32_t inter, void* act,
-                                       void* y, void*, size_t, void* stream) {
+                                       void* y, int32_t phases, void*, size_t, void* stream) {
     return moe::grouped_swiglu<false>(x, row_map, w_gate, w_up, w_down, nullptr, nullptr, nullptr, offsets, n_rows,
-                                      n_experts, hidden, inter, act, y, stream, "moe_grouped_swiglu_bf16");
+                                      n_experts, hidden, inter, act, y, phases, stream, "moe_grouped_swiglu_bf16");
 }
 
 extern "C" int moe_grouped_swiglu_w8a16(const void* x, const int32_t* row_map, const void* const* w_gate,
                                         const void* const* w_up, const void* const* w_down,
                                         const float* const* s_gate, const float* const* s_up,
                                         const float* const* s_down, const int32_t* offsets, int32_t n_rows,
-                                        int32_t n_experts, int32_t hidden, int32_t inter, void* act, void* y, void*,
-                                        size_t, void* stream) {
+                                        int32_t n_experts, int32_t hidden, int32_t inter, void* act, void* y,
+                                        int32_t phases, void*, size_t, void* stream) {
     return moe::grouped_swiglu<true>(x, row_map, w_gate, w_up, w_down, s_gate, s_up, s_down, offsets, n_rows,
-                                     n_experts, hidden, inter, act, y, stream, "moe_grouped_swiglu_w8a16");
+                                     n_experts, hidden, inter, act, y, phases, stream, "moe_grouped_swiglu_w8a16");
 }
 
 extern "C" int moe_dequant_fp8_block128(const void* q, const float* scale, int32_t rows, int32_t cols, void* out,

@@ -148,8 +148,11 @@ def expert_pointers(gates, ups, downs, s_gates=None, s_ups=None, s_downs=None, d
     return ExpertPointers(E, h, I, fp8, table(gates), table(ups), table(downs), sg, su, sd, keep)
 
 
+PHASE_GATE_UP, PHASE_DOWN, PHASE_BOTH = 1, 2, 3
+
+
 def grouped_swiglu(x: torch.Tensor, row_map, ptrs: ExpertPointers, offsets: torch.Tensor, n_rows: int,
-                   act: torch.Tensor | None = None, y: torch.Tensor | None = None):
+                   act: torch.Tensor | None = None, y: torch.Tensor | None = None, phases: int = PHASE_BOTH):
     """All experts' SwiGLU MLPs on their row ranges.  x: bf16 sorted rows [n_rows,h], or the
     unsorted matrix with row_map int32 [n_rows].  Returns y bf16 [n_rows,h] (sorted-row order)."""
     _need(x, torch.bfloat16, "x")
@@ -173,11 +176,11 @@ def grouped_swiglu(x: torch.Tensor, row_map, ptrs: ExpertPointers, offsets: torc
         N.check(L.moe_grouped_swiglu_w8a16(_ptr(x), _ptr(row_map), _ptr(ptrs.w_gate), _ptr(ptrs.w_up),
                                            _ptr(ptrs.w_down), _ptr(ptrs.s_gate), _ptr(ptrs.s_up),
                                            _ptr(ptrs.s_down), _ptr(offsets), n_rows, E, h, I, _ptr(act), _ptr(y),
-                                           None, 0, _stream()), "moe_grouped_swiglu_w8a16")
+                                           phases, None, 0, _stream()), "moe_grouped_swiglu_w8a16")
     else:
         N.check(L.moe_grouped_swiglu_bf16(_ptr(x), _ptr(row_map), _ptr(ptrs.w_gate), _ptr(ptrs.w_up),
                                           _ptr(ptrs.w_down), _ptr(offsets), n_rows, E, h, I, _ptr(act), _ptr(y),
-                                          None, 0, _stream()), "moe_grouped_swiglu_bf16")
+                                          phases, None, 0, _stream()), "moe_grouped_swiglu_bf16")
     return y
 
 
