@@ -63,10 +63,11 @@ class MoEGate(nn.Module):
         if self.training:
             raise NotImplementedError("inference only: the auxiliary loss is not computed")
         from .block import _gate_weight_bf16
+        spec = _spec(self)
         h = hidden_states.shape[-1]
         x = hidden_states.reshape(-1, h)
         cache = self.__dict__.setdefault("_moe_cache", {})
-        idx, w, _ = ops.router(x.contiguous(), _gate_weight_bf16(self.weight, cache), None, _spec(self))
+        idx, w, _ = ops.router(x.contiguous(), _gate_weight_bf16(self.weight, cache), None, spec)
         return idx.to(torch.int64), w, None
 
 

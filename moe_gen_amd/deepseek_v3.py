@@ -62,11 +62,12 @@ class MoEGate(nn.Module):
         """-> (topk_idx int64 [n,k], topk_weight fp32 [n,k]); slots in descending score."""
         assert not self.training
         from .block import _gate_weight_bf16
+        spec = _spec(self)
         h = hidden_states.shape[-1]
         x = hidden_states.reshape(-1, h)
         cache = self.__dict__.setdefault("_moe_cache", {})
         idx, w, _ = ops.router(x.contiguous(), _gate_weight_bf16(self.weight, cache),
-                               self.e_score_correction_bias.data.to(torch.float32), _spec(self))
+                               self.e_score_correction_bias.data.to(torch.float32), spec)
         return idx.to(torch.int64), w
 
 

@@ -126,3 +126,11 @@ def test_fp8_decode_table_on_device():
     tab = O.fp8_table()
     ok = ~np.isnan(tab)
     assert np.array_equal(out[ok], tab[ok]) and np.isnan(out[~ok]).all()
+
+
+def test_dequant_golden_fixture():
+    import os
+    from moe_gen_amd import ops
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", "fp8_dequant.npz"))
+    out = ops.dequant_fp8_block128(torch.from_numpy(z["q"]).cuda().view(torch.float8_e4m3fn), torch.from_numpy(z["scale"]).cuda())
+    assert np.array_equal(bits(out), z["out"])

@@ -100,3 +100,22 @@ def test_canonical_exp_sigmoid_on_device():
         assert np.array_equal(lg.view(np.uint32), ol.view(np.uint32))
         assert np.array_equal(idx, oi)
         assert np.array_equal(w.view(np.uint32), ow.view(np.uint32))
+
+
+def test_router_and_dispatch_golden_fixtures():
+    """The committed vectors (tests/golden/router_*.npz) through the C ABI."""
+    import glob
+    import os
+    from moe_gen_amd import ops
+    from util import bf16_tensor
+    files = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "router_*.npz")))
+    assert len(files) >= 4
+    for f in files:
+        z = np.load(f)
+        spec = O.RouterSpec(**{k[5:]: z[k].item() for k in z.files if k.startswith("spec_")})
+        bias = torch.from_numpy(z["bias"]) if "bias" in z.files else None
+        idx, w, _ = gpu_router(bf16_tensor(z["x"]), bf16_tensor(z["gate"]), bias, spec)
+        assert np.array_equal(idx, z["idx"]) and np.array_equal(w.view(np.uint32), z["w"].view(np.uint32)), f
+        counts, offsets, perm, pos, _ = ops.dispatch(torch.from_numpy(idx).cuda(), spec.n_experts)
+        assert np.array_equal(counts.cpu().numpy(), z["counts"]) and np.array_equal(perm.cpu().numpy(), z["perm"])
+        assert np.array_equal(offsets.cpu().numpy(), z["offsets"]) and np.array_equal(pos.cpu().numpy(), z["pos"])
