@@ -20,16 +20,19 @@
 // so that each XCD owns a contiguous range of tiles (same expert, neighbouring M/N
 // tiles), which is what makes its private L2 hold the A and B panels that are re-read.
 //
-// Workgroup = 4 waves (2 along M, 2 along N).  Per wave MT x 4 MFMA tiles of 32x32
-// (v_mfma_f32_32x32x16_bf16), i.e. up to 128x128 outputs and 256 fp32 accumulators.
-// K advances 64 at a time through a double-buffered LDS stage; rows are 128 bytes with a
-// 16-byte-chunk XOR swizzle (chunk ^= row & 7) so that both the 16-byte stores and the
-// 16-byte MFMA operand reads are bank-conflict free.  Global loads for stage k+2 are in
-// flight while stage k is multiplied.
+// Workgroup = 8 waves (2 along M, 4 along N), two per SIMD.  Per wave MT x 2 MFMA tiles of
+// 32x32 (v_mfma_f32_32x32x16_bf16), i.e. up to 128x64 outputs and 128 fp32 accumulators.
+// K advances 64 at a time through two LDS stages; rows are 128 bytes with a 16-byte-chunk
+// XOR swizzle so that both the 16-byte stores and the 16-byte MFMA operand reads are
+// bank-conflict free.  Global loads for tile k+2 are in flight while tile k is multiplied
+// and tile k+1 is written to LDS.  The two waves of a SIMD run the halves of an iteration
+// (MFMA work / data movement) in opposite order, so the matrix core and the LDS port are
+// both kept busy between the one barrier per k-stage.
 //
 // The MFMA is issued with the WEIGHT fragment as srcA and the TOKEN fragment as srcB, so
 // a lane ends up holding 4 consecutive output columns of one token row per register
 // quad: the epilogue packs them into one 8-byte store.
+
 #include "common.h"
 
 namespace moe {
@@ -75,24 +78,57 @@ struct GemmArgs {
     int n_tiles_n;              // ceil(N / (SWIGLU ? 128 : 256))
 };
 
-template <int MT, bool SWIGLU, bool W8>
-__global__ __launch_bounds__(256) void grouped_gemm_kernel(GemmArgs g) {
+// LDS rows are 128 bytes = 8 chunks of 16 bytes; chunk c of row r is stored at chunk c ^ swz(r).
+// swz makes any 8 consecutive rows hit 8 different chunks (32 banks x 4 B = one 128-byte row per
+// cycle) AND any 16 consecutive rows hit 16 different (row parity, chunk) slots (64 banks =
+// two rows per cycle), so 16-byte operand reads by 32 consecutive rows never collide.
+__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+// global-address-space views: expert pointers come out of a pointer table in memory, and
+// without the address space the compiler must emit flat loads, whose completion is tracked
+// by the same counter as the LDS reads of the MFMA operands
+typedef const __attribute__((address_space(1))) u32x4* gptr_u32x4;
+typedef const __attribute__((address_space(1))) float* gptr_f32;
+typedef const __attribute__((address_space(1))) int32_t* gptr_i32;
+
+__device__ __forceinline__ u32x4 gload16(const void* p) { return *(gptr_u32x4)(uintptr_t)p; }
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ const uint8_t* uni_ptr(const void* p) {
+    uint64_t u = (uint64_t)(uintptr_t)p;
+    uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)u), hi = __builtin_amdgcn_readfirstlane((uint32_t)(u >> 32));
+    return reinterpret_cast<const uint8_t*>((uintptr_t)(((uint64_t)hi << 32) | lo));
+}
+
+// MT: 32-row MFMA tiles per wave along M (workgroup rows BM = 64*MT, 2 waves along M)
+// WN: waves along N; 4 -> 8 waves of up to 128x64 outputs, two per SIMD, which issue their MFMA
+//     half and their load/dequantise/store half of an iteration in opposite order, so that one
+//     feeds the matrix core while the other feeds LDS
+template <int MT, int WN, bool SWIGLU, bool W8>
+__global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
+    constexpr int NT = 128 * WN;                // threads
     constexpr int BM = 64 * MT;                 // rows per workgroup
     constexpr int A_STAGE = BM * ROW_B;         // bytes
     constexpr int B_STAGE = BN_ROWS * ROW_B;
-    constexpr int NA = MT * 2;                  // 16-byte A chunks per thread per stage
-    constexpr int NB = W8 ? 4 : 8;              // 16-byte global B chunks per thread per stage
+    constexpr int RA = NT / 8;                  // A rows covered by one pass of the workgroup
+    constexpr int NA = BM / RA;                 // 16-byte A chunks per thread per stage
+    constexpr int RB = W8 ? NT / 4 : NT / 8;    // B rows per pass (fp8 rows are 4 chunks of 16 weights)
+    constexpr int NB = BN_ROWS / RB;            // 16-byte global B chunks per thread per stage
     constexpr int NBLK = SWIGLU ? 128 : 256;    // output columns per workgroup
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    constexpr int NJ = 8 / WN;                  // 32-wide weight tiles per wave
+    static_assert(NA >= 1 && NB >= 2, "tile/thread mismatch");
+    // two separate arrays: stores into one stage and reads from the other provably do not alias,
+    // which lets the scheduler move them past each other
+    __shared__ __attribute__((aligned(16))) uint8_t smem0[A_STAGE + B_STAGE];
+    __shared__ __attribute__((aligned(16))) uint8_t smem1[A_STAGE + B_STAGE];
     __shared__ int s_pref[MAX_E + 1];
-    __shared__ int s_wtot[4];
+    __shared__ int s_wtot[NT / 64];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave & 1, wn = wave >> 1;
+    const int wm = wave & 1, wn = (wave >> 1) % WN;
 
     // ---- M-tile prefix over experts (exclusive scan of ceil(count/BM)) ----
     int run = 0;
-    for (int e0 = 0; e0 < g.E; e0 += 256) {
+    for (int e0 = 0; e0 < g.E; e0 += NT) {
         int e = e0 + tid;
         int mt = 0;
         if (e < g.E) mt = (g.offsets[e + 1] - g.offsets[e] + BM - 1) / BM;
@@ -104,10 +140,14 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(GemmArgs g) {
         }
         if (lane == 63) s_wtot[wave] = inc;
         __syncthreads();
-        int pre = run;
-        for (int w = 0; w < wave; ++w) pre += s_wtot[w];
+        int pre = run, tot = 0;
+#pragma unroll
+        for (int w = 0; w < NT / 64; ++w) {
+            if (w < wave) pre += s_wtot[w];
+            tot += s_wtot[w];
+        }
         if (e < g.E) s_pref[e] = pre + inc - mt;
-        run += s_wtot[0] + s_wtot[1] + s_wtot[2] + s_wtot[3];
+        run += tot;
         __syncthreads();
     }
     if (tid == 0) s_pref[g.E] = run;
@@ -125,47 +165,51 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(GemmArgs g) {
         int mid = (lo + hi) >> 1;
         if (s_pref[mid] <= q) lo = mid; else hi = mid;
     }
-    const int e = lo;
-    const int mt_e = s_pref[e + 1] - s_pref[e];
-    const int local = v - s_pref[e] * g.n_tiles_n;
+    const int e = uni(lo);
+    const int pe = uni(s_pref[e]);
+    const int mt_e = uni(s_pref[e + 1]) - pe;
+    const int local = v - pe * g.n_tiles_n;
     const int n_tile = local / mt_e, m_tile = local - n_tile * mt_e;
-    const int row0 = g.offsets[e] + m_tile * BM;
-    const int row_end = g.offsets[e + 1];
+    const int row0 = uni(g.offsets[e]) + m_tile * BM;
+    const int row_end = uni(g.offsets[e + 1]);
     const int n0 = n_tile * NBLK;
     const int K = g.K, N = g.N;
 
     // ---- per-thread load coordinates ----
-    const int lrow = tid >> 3, lchunk = tid & 7;          // bf16 tiles: row tid/8 (+32 i), chunk tid%8
+    const int lrow = tid >> 3, lchunk = tid & 7;          // bf16 tiles: row tid/8 (+RA i), chunk tid%8
     int a_src[NA];
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
-        int r = min(row0 + lrow + 32 * i, row_end - 1);
-        a_src[i] = g.row_map ? g.row_map[r] : r;
+        int r = min(row0 + lrow + RA * i, row_end - 1);
+        a_src[i] = g.row_map ? ((gptr_i32)(uintptr_t)g.row_map)[r] : r;
     }
-    const uint32_t a_lds = (uint32_t)(lrow * ROW_B + ((lchunk ^ (lrow & 7)) << 4));
+    const uint32_t a_lds = (uint32_t)(lrow * ROW_B + ((lchunk ^ swz(lrow)) << 4));
 
-    const uint8_t* bmat0 = static_cast<const uint8_t*>(g.b0[e]);
-    const uint8_t* bmat1 = SWIGLU ? static_cast<const uint8_t*>(g.b1[e]) : bmat0;
-    const float* sc0 = W8 ? g.s0[e] : nullptr;
-    const float* sc1 = (W8 && SWIGLU) ? g.s1[e] : sc0;
+    const uint8_t* bmat0 = uni_ptr(g.b0[e]);
+    const uint8_t* bmat1 = SWIGLU ? uni_ptr(g.b1[e]) : bmat0;
+    gptr_f32 sc0 = W8 ? (gptr_f32)(uintptr_t)uni_ptr(g.s0[e]) : nullptr;
+    gptr_f32 sc1 = (W8 && SWIGLU) ? (gptr_f32)(uintptr_t)uni_ptr(g.s1[e]) : sc0;
     constexpr int EB = W8 ? 1 : 2;                        // bytes per weight element
-    const int brow = W8 ? (tid >> 2) : (tid >> 3);        // fp8 tiles: row tid/4 (+64 i), 16-byte chunk tid%4
+    const int brow = W8 ? (tid >> 2) : (tid >> 3);        // fp8 tiles: row tid/4 (+RB i), 16-byte chunk tid%4
     const int bcol_b = W8 ? ((tid & 3) << 4) : ((tid & 7) << 4);  // byte offset inside the 64-element k slab
-    constexpr int BSTEP = W8 ? 64 : 32;                   // row step between a thread's B chunks
     int b_n[NB];
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
-        int r = brow + BSTEP * i;                         // row inside the 256-row B tile
+        int r = brow + RB * i;                            // row inside the 256-row B tile
         int n = SWIGLU ? (n0 + (r & 127)) : (n0 + r);
         b_n[i] = min(n, N - 1);
     }
     uint32_t b_lds[2];
+    // fp8: a thread owns chunks 2q and 2q+1 of its row; rows with bit 1 set store them in the
+    // opposite order so that the 16 lanes of one store instruction (4 rows x 4 chunks) spread
+    // over all banks
+    const bool b_swap = W8 && ((brow >> 1) & 1);
     if (W8) {
-        int qd = tid & 3, sw = brow & 7;
-        b_lds[0] = (uint32_t)(brow * ROW_B + (((2 * qd) ^ sw) << 4));
-        b_lds[1] = (uint32_t)(brow * ROW_B + (((2 * qd + 1) ^ sw) << 4));
+        int qd = tid & 3, sw = swz(brow), first = b_swap ? 1 : 0;
+        b_lds[0] = (uint32_t)(brow * ROW_B + (((2 * qd + first) ^ sw) << 4));
+        b_lds[1] = (uint32_t)(brow * ROW_B + (((2 * qd + 1 - first) ^ sw) << 4));
     } else {
-        b_lds[0] = (uint32_t)(brow * ROW_B + (((tid & 7) ^ (brow & 7)) << 4));
+        b_lds[0] = (uint32_t)(brow * ROW_B + (((tid & 7) ^ swz(brow)) << 4));
         b_lds[1] = 0;
     }
     // block-scale rows (W8): first / second 128 rows of the B tile
@@ -176,90 +220,113 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(GemmArgs g) {
         else        { srow0 = (n0 >> 7) * KB; srow1 = min((n0 >> 7) + 1, (N >> 7) - 1) * KB; }
     }
 
-    u32x4 ra[NA], rb[NB];
-    float rs[2] = {1.0f, 1.0f};
+    u32x4 ra[1][NA], rb[1][NB];
+    float rs[1][2] = {{1.0f, 1.0f}};
+    constexpr int set = 0;
     auto gload = [&](int kt) {
         const size_t kofs = (size_t)kt * BK;
 #pragma unroll
-        for (int i = 0; i < NA; ++i)
-            ra[i] = *reinterpret_cast<const u32x4*>(g.a + (size_t)a_src[i] * K + kofs + lchunk * 8);
+        for (int i = 0; i < NA; ++i) ra[set][i] = gload16(g.a + (size_t)a_src[i] * K + kofs + lchunk * 8);
 #pragma unroll
         for (int i = 0; i < NB; ++i) {
             const uint8_t* m = (SWIGLU && i >= NB / 2) ? bmat1 : bmat0;  // rows >= 128 of the B tile are the up matrix
-            rb[i] = *reinterpret_cast<const u32x4*>(m + ((size_t)b_n[i] * K + kofs) * EB + bcol_b);
+            rb[set][i] = gload16(m + ((size_t)b_n[i] * K + kofs) * EB + bcol_b);
         }
         if (W8) {
-            rs[0] = sc0[srow0 + (kt >> 1)];
-            rs[1] = sc1[srow1 + (kt >> 1)];
+            rs[set][0] = sc0[srow0 + (kt >> 1)];
+            rs[set][1] = sc1[srow1 + (kt >> 1)];
         }
     };
-    auto lds_store = [&](int stage) {
-        uint8_t* As = smem + stage * (A_STAGE + B_STAGE);
+    auto lds_store = [&](uint8_t* As) {
         uint8_t* Bs = As + A_STAGE;
 #pragma unroll
-        for (int i = 0; i < NA; ++i) *reinterpret_cast<u32x4*>(As + a_lds + i * 32 * ROW_B) = ra[i];
+        for (int i = 0; i < NA; ++i) *reinterpret_cast<u32x4*>(As + a_lds + i * RA * ROW_B) = ra[set][i];
         if (W8) {
 #pragma unroll
             for (int i = 0; i < NB; ++i) {
                 u32x4 l, h;
-                dequant16(rb[i], rs[i >> 1], l, h);
-                *reinterpret_cast<u32x4*>(Bs + b_lds[0] + i * 64 * ROW_B) = l;
-                *reinterpret_cast<u32x4*>(Bs + b_lds[1] + i * 64 * ROW_B) = h;
+                dequant16(rb[set][i], rs[set][i / (NB / 2)], l, h);
+                *reinterpret_cast<u32x4*>(Bs + b_lds[0] + i * RB * ROW_B) = b_swap ? h : l;
+                *reinterpret_cast<u32x4*>(Bs + b_lds[1] + i * RB * ROW_B) = b_swap ? l : h;
             }
         } else {
 #pragma unroll
-            for (int i = 0; i < NB; ++i) *reinterpret_cast<u32x4*>(Bs + b_lds[0] + i * 32 * ROW_B) = rb[i];
+            for (int i = 0; i < NB; ++i) *reinterpret_cast<u32x4*>(Bs + b_lds[0] + i * RB * ROW_B) = rb[set][i];
         }
     };
 
     // ---- MFMA operand coordinates ----
-    // fragment row = base + lane%32; logical chunk = 2*s + lane/32; swizzle key = lane%8
-    const int frow = lane & 31, fhalf = lane >> 5, fkey = lane & 7;
-    uint32_t tok_off[MT], w_off[4];
+    // fragment row = base + lane%32 (bases are multiples of 32); logical chunk = 2*s + lane/32
+    const int frow = lane & 31, fhalf = lane >> 5, fkey = swz(frow);
+    uint32_t tok_off[MT], w_off[NJ];
 #pragma unroll
     for (int mi = 0; mi < MT; ++mi) tok_off[mi] = (uint32_t)((wm * 32 * MT + 32 * mi + frow) * ROW_B);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        int r = SWIGLU ? ((j < 2 ? 0 : 128) + wn * 64 + 32 * (j & 1)) : (wn * 128 + 32 * j);
+    for (int j = 0; j < NJ; ++j) {
+        int r = SWIGLU ? ((j < NJ / 2 ? 0 : 128) + wn * (16 * NJ) + 32 * (j % (NJ / 2))) : (wn * (32 * NJ) + 32 * j);
         w_off[j] = (uint32_t)((r + frow) * ROW_B);
     }
 
-    f32x16 acc[MT][4];
+    f32x16 acc[MT][NJ];
 #pragma unroll
     for (int mi = 0; mi < MT; ++mi)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[mi][j] = f32x16{0};
+        for (int j = 0; j < NJ; ++j) acc[mi][j] = f32x16{0};
 
-    auto compute = [&](int stage) {
-        const uint8_t* As = smem + stage * (A_STAGE + B_STAGE);
+    // Operand fragments are double-buffered in registers: the 16-byte LDS reads of k-step s+1
+    // are issued before the MFMAs of k-step s.
+    auto compute = [&](const uint8_t* As) {
         const uint8_t* Bs = As + A_STAGE;
+        bf16x8 tf[2][MT], wf[2][NJ];
+        auto read_frags = [&](int s, int buf) {
+            const uint32_t coff = (uint32_t)(((2 * s + fhalf) ^ fkey) << 4);
+#pragma unroll
+            for (int mi = 0; mi < MT; ++mi) tf[buf][mi] = *reinterpret_cast<const bf16x8*>(As + tok_off[mi] + coff);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) wf[buf][j] = *reinterpret_cast<const bf16x8*>(Bs + w_off[j] + coff);
+        };
+        read_frags(0, 0);
 #pragma unroll
         for (int s = 0; s < BK / 16; ++s) {
-            const uint32_t coff = (uint32_t)(((2 * s + fhalf) ^ fkey) << 4);
-            bf16x8 tf[MT], wf[4];
-#pragma unroll
-            for (int mi = 0; mi < MT; ++mi) tf[mi] = *reinterpret_cast<const bf16x8*>(As + tok_off[mi] + coff);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) wf[j] = *reinterpret_cast<const bf16x8*>(Bs + w_off[j] + coff);
+            if (s + 1 < BK / 16) read_frags(s + 1, (s + 1) & 1);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int mi = 0; mi < MT; ++mi)
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    acc[mi][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[j], tf[mi], acc[mi][j], 0, 0, 0);
+                for (int j = 0; j < NJ; ++j)
+                    acc[mi][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[s & 1][j], tf[s & 1][mi], acc[mi][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
     // ---- main loop ----
+    // On entry to iteration kt: LDS stage kt&1 holds tile kt and the registers hold tile kt+1
+    // (possibly still in flight).  The iteration moves tile kt+1 into the other LDS stage, refills
+    // the registers with tile kt+2 and multiplies tile kt.
     const int nk = K / BK;
     gload(0);
-    lds_store(0);
+    lds_store(smem0);
     if (nk > 1) gload(1);
     __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-        const int cur = kt & 1;
-        if (kt + 1 < nk) lds_store(cur ^ 1);
-        if (kt + 2 < nk) gload(kt + 2);
-        compute(cur);
+    int kt = 0;
+    const bool mfma_first = wave < 4;   // waves w and w+4 share a SIMD
+    for (; kt < nk; ++kt) {
+        const uint8_t* rd = (kt & 1) ? smem1 : smem0;
+        uint8_t* wr = (kt & 1) ? smem0 : smem1;
+        // the wave that is multiplying outranks its SIMD partner that is moving data
+        if (mfma_first) {
+            __builtin_amdgcn_s_setprio(2);
+            compute(rd);
+            __builtin_amdgcn_s_setprio(0);
+            if (kt + 1 < nk) lds_store(wr);
+            if (kt + 2 < nk) gload(kt + 2);
+        } else {
+            if (kt + 1 < nk) lds_store(wr);
+            if (kt + 2 < nk) gload(kt + 2);
+            __builtin_amdgcn_s_setprio(2);
+            compute(rd);
+            __builtin_amdgcn_s_setprio(0);
+        }
         __syncthreads();
     }
 
@@ -274,15 +341,15 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(GemmArgs g) {
         uint16_t* crow = g.c + (size_t)(row0 + ml) * N;
         if (SWIGLU) {
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
+            for (int j = 0; j < NJ / 2; ++j) {
 #pragma unroll
                 for (int qd = 0; qd < 4; ++qd) {
-                    const int n = n0 + wn * 64 + 32 * j + 8 * qd + 4 * fhalf;
+                    const int n = n0 + wn * (16 * NJ) + 32 * j + 8 * qd + 4 * fhalf;
                     float o[4];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         float gv = bf16r(acc[mi][j][4 * qd + i]);
-                        float uv = bf16r(acc[mi][j + 2][4 * qd + i]);
+                        float uv = bf16r(acc[mi][j + NJ / 2][4 * qd + i]);
                         float sg = bf16r(gv * __builtin_amdgcn_rcpf(1.0f + __expf(-gv)));
                         o[i] = sg * uv;
                     }
@@ -294,10 +361,10 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(GemmArgs g) {
             }
         } else {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < NJ; ++j) {
 #pragma unroll
                 for (int qd = 0; qd < 4; ++qd) {
-                    const int n = n0 + wn * 128 + 32 * j + 8 * qd + 4 * fhalf;
+                    const int n = n0 + wn * (32 * NJ) + 32 * j + 8 * qd + 4 * fhalf;
                     if (n < N) {
                         u32x2 pk = {pack_bf16(acc[mi][j][4 * qd], acc[mi][j][4 * qd + 1]),
                                     pack_bf16(acc[mi][j][4 * qd + 2], acc[mi][j][4 * qd + 3])};
@@ -309,24 +376,17 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(GemmArgs g) {
     }
 }
 
-template <int MT, bool SWIGLU, bool W8>
+template <int MT, int WN, bool SWIGLU, bool W8>
 int launch_one(const GemmArgs& g, int n_rows, hipStream_t st) {
     constexpr int BM = 64 * MT;
-    constexpr int LDS = 2 * (BM * ROW_B + BN_ROWS * ROW_B);
-    static bool attr_set = false;
-    auto kern = grouped_gemm_kernel<MT, SWIGLU, W8>;
-    if (!attr_set) {
-        MOE_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
-        attr_set = true;
-    }
+    auto kern = grouped_gemm_kernel<MT, WN, SWIGLU, W8>;
     const long max_mtiles = (long)n_rows / BM + g.E;  // sum_e ceil(c_e/BM) <= n_rows/BM + E
     const long grid = ((max_mtiles * g.n_tiles_n + 7) / 8) * 8;
     if (grid > 0x7fffffffL) {
         set_error("grouped gemm: %ld workgroups exceed the grid limit", grid);
         return MOE_ERR_INVALID;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), LDS, st, g);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(128 * WN), 0, st, g);
     MOE_HIP_CHECK(hipGetLastError());
     return MOE_OK;
 }
@@ -334,9 +394,9 @@ int launch_one(const GemmArgs& g, int n_rows, hipStream_t st) {
 template <bool SWIGLU, bool W8>
 int launch_mt(const GemmArgs& g, int n_rows, hipStream_t st) {
     const long mean = g.E > 0 ? (long)n_rows / g.E : 0;
-    if (mean >= 192) return launch_one<4, SWIGLU, W8>(g, n_rows, st);
-    if (mean >= 96) return launch_one<2, SWIGLU, W8>(g, n_rows, st);
-    return launch_one<1, SWIGLU, W8>(g, n_rows, st);
+    if (mean >= 192) return launch_one<4, 4, SWIGLU, W8>(g, n_rows, st);
+    if (mean >= 96) return launch_one<2, 4, SWIGLU, W8>(g, n_rows, st);
+    return launch_one<1, 4, SWIGLU, W8>(g, n_rows, st);
 }
 
 template <bool W8>
