@@ -61,35 +61,96 @@ def cpu_baseline(w, blk, n_sample: int):
                       f"({dt:.1f} s); stock-PyTorch CPU restatement of the reference block"}
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="deepseek_v3_w8a16")
-    ap.add_argument("--tokens", type=int, default=0, help="override the token count (parity/debug only)")
-    ap.add_argument("--materialize", action="store_true", help="gather rows into a sorted copy instead of "
-                    "reading them through the row map inside the GEMM")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample", type=int, default=128)
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); use --gpus 1")
+def staged_run(w, blk, x, steps: int):
+    """Second figure: the same block with every expert matrix in pinned host memory, delivered by
+    the stager (cyclic prefetch on the copy stream, event hand-off) while the previous layer
+    computes.  Two layers' worth of modules alternate so that copies overlap compute, as in a model."""
+    import time as _t
 
+    import torch
+    from moe_gen_amd import StagedExpert, Stager
+
+    E = w.E
+    wdt = torch.float8_e4m3fn if w.fp8 else torch.bfloat16
+    names = blk.experts[0].names
+    shapes = {"routed_expert": {f"{n}.weight": (tuple(getattr(blk.experts[0], n).weight.shape), wdt) for n in names}}
+    n_slots = {"routed_expert": 2 * E}
+    has_shared = bool(w.S) and w.family != "mixtral"
+    if has_shared:
+        shapes["shared_expert"] = {f"{n}.weight": (tuple(getattr(blk.shared_experts, n).weight.shape), wdt) for n in names}
+        n_slots["shared_expert"] = 2
+    st = Stager(shapes, n_slots, device="cuda:0", model_type={"v3": "deepseek_v3", "v2": "deepseek_v2"}.get(w.family, "mixtral"),
+                num_hidden_layers=64, num_local_experts=E)
+    layers = (10, 11)
+
+    def scales_of(mlp):
+        if not w.fp8:
+            return None
+        return {f"{n}.weight_scale_inv": getattr(mlp, n).weight_scale_inv.data for n in names}
+
+    staged = {}
+    host = {}
+    for e in range(E):
+        host[e] = {f"{n}.weight": getattr(blk.experts[e], n).weight.data.cpu().pin_memory() for n in names}
+    if has_shared:
+        host["s"] = {f"{n}.weight": getattr(blk.shared_experts, n).weight.data.cpu().pin_memory() for n in names}
+    for L in layers:
+        for e in range(E):
+            st.add_module(f"routed_expert_{L}_{e}", "routed_expert", host[e])
+        if has_shared:
+            st.add_module(f"shared_expert_{L}", "shared_expert", host["s"])
+        staged[L] = ([StagedExpert(blk.experts[e], L, e, st, scales_of(blk.experts[e])) for e in range(E)],
+                     StagedExpert(blk.shared_experts, L, -1, st, scales_of(blk.shared_experts)) if has_shared else None)
+    resident_experts = blk.experts
+    resident_shared = blk.shared_experts if has_shared else None
+    import torch.nn as nn
+
+    def step(i):
+        ex, sh = staged[layers[i % 2]]
+        blk.experts = nn.ModuleList(ex)
+        if has_shared:
+            blk.shared_experts = sh
+        return blk(x)
+
+    st.pump()
+    step(0); step(1)
+    torch.cuda.synchronize()
+    t0 = _t.perf_counter()
+    for i in range(steps):
+        step(i)
+    torch.cuda.synchronize()
+    dt = _t.perf_counter() - t0
+    copies, nbytes = st.stats()
+    blk.experts = resident_experts
+    if has_shared:
+        blk.shared_experts = resident_shared
+    st.close()
+    return {"tokens_per_s": w.n * steps / dt, "ms_per_step": dt * 1e3 / steps,
+            "host_to_hbm_gib_per_step": nbytes / copies * (E + (1 if has_shared else 0)) / 2 ** 30,
+            "note": "all expert weights re-staged from pinned host memory every step (the reference's policy); "
+                    "bounded by the host link, not by the kernels"}
+
+
+# HBM traffic per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (two runs; FETCH_SIZE scaled by 2.0, the factor a plain copy kernel of known size showed on this
+# box, WRITE_SIZE by 1.0).  bench.py cannot run the profiler on itself, so the figures are recorded
+# here from profiles/ for the workloads that were profiled; None elsewhere.
+MEASURED_TRAFFIC_BYTES = {"deepseek_v3_w8a16": 26.5e9}   # profiles/pmc_traffic_deepseek_v3_w8a16_65536.md
+
+
+def run_workload(name: str, args, with_cpu: bool):
     import torch
     from moe_gen_amd import synthetic
     from moe_gen_amd.block import StageTimer
 
-    w = synthetic.WORKLOADS[args.workload]
+    w = synthetic.WORKLOADS[name]
     if args.tokens:
         w = w.scaled(n=args.tokens)
     dev = "cuda:0"
-    torch.cuda.set_device(0)
     blk = synthetic.build_block(w, device=dev, gen_device=dev)
     blk.fused_gather = not args.materialize
     x = synthetic.hidden_states(w, dev)
     torch.cuda.synchronize()
-
     for _ in range(args.warmup):
         blk(x)
     torch.cuda.synchronize()
@@ -107,9 +168,9 @@ def main():
     tokens_per_s = w.n * args.steps / dt
 
     st = {k: sum(v) / len(v) for k, v in timer.totals_ms().items()}
-    # dominant kernel: the fused gate/up SwiGLU GEMM.  It is launched once for the routed experts
-    # and once for the shared expert per step (same kernel, different row counts): algorithmic FLOP
-    # per launch and average launch duration are both averages over those launches.
+    # dominant kernel: the fused gate/up SwiGLU GEMM.  With shared experts it is launched twice per
+    # step (routed experts, shared expert; same kernel, different row counts): algorithmic FLOP per
+    # launch and average launch duration are both averages over those launches.
     gu_flop = [4.0 * w.n * w.k * w.h * w.I]
     gu_ms = [st["routed_gate_up"]]
     if "shared_gate_up" in st:
@@ -121,23 +182,29 @@ def main():
     gemm_ms = sum(st.get(k, 0.0) for k in ("routed_gate_up", "routed_down", "shared_gate_up", "shared_down"))
     gemm_tflops = (w.routed_flop + w.shared_flop) / (gemm_ms * 1e-3) / 1e12
     disp_bytes = w.dispatch_bytes if args.materialize else 4.0 * w.n * w.k
+    mean_rows = w.n * w.k // w.E
+    mt = 4 if mean_rows >= 192 else (2 if mean_rows >= 96 else 1)
+    wbytes = 3.0 * w.E * w.h * w.I * (1 if w.fp8 else 2)
     result = {
-        "metric": "MoE-layer tokens/sec at DeepSeek-V3 W8A16 shape" if args.workload == "deepseek_v3_w8a16"
-                  else f"MoE-layer tokens/sec ({args.workload})",
+        "metric": "MoE-layer tokens/sec at DeepSeek-V3 W8A16 shape" if name == "deepseek_v3_w8a16"
+                  else f"MoE-layer tokens/sec ({name})",
         "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16",
-        "data": "synthetic",
+        "dtype": "bf16", "data": "synthetic",
         "config": {"workload": w.name, "tokens": w.n, "hidden": w.h, "experts": w.E, "top_k": w.k,
-                   "moe_intermediate": w.I, "shared_experts": w.S, "weights": "fp8-e4m3fn+128x128 fp32 scales" if w.fp8 else "bf16",
+                   "moe_intermediate": w.I, "shared_experts": w.S,
+                   "weights": "fp8-e4m3fn + 128x128 fp32 scales, dequantised to bf16 ahead of MFMA" if w.fp8 else "bf16",
                    "gather": "materialized" if args.materialize else "fused into the GEMM A-operand load"},
-        "roofline": {"bound": "mfma", "kernel": "grouped_gemm_kernel<MT=4,SWIGLU,W8> (gate/up + SiLU*mul)",
+        "roofline": {"bound": "mfma",
+                     "kernel": f"grouped_gemm_kernel<MT={mt},WN=4,SWIGLU=true,W8={'true' if w.fp8 else 'false'}> (gate/up + SiLU*mul)",
                      "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(name),
                      "frac_of_fp8_peak": achieved / PEAK_FP8_TFLOPS,
-                     "launches_per_step": len(gu_ms), "avg_launch_ms": ms_per_launch},
+                     "launches_per_step": len(gu_ms), "avg_launch_ms": ms_per_launch,
+                     "flop_per_launch": flop_per_launch},
         "pct_mfma_peak": {"all_expert_gemms_tflops": gemm_tflops, "of_bf16_peak": gemm_tflops / PEAK_BF16_TFLOPS,
-                          "of_fp8_peak": gemm_tflops / PEAK_FP8_TFLOPS},
+                          "of_fp8_peak": gemm_tflops / PEAK_FP8_TFLOPS,
+                          "weight_stream_gbps": wbytes / (gemm_ms * 1e-3) / 1e9},
         "routing_gbps": {"router": w.router_bytes / (st["router"] * 1e-3) / 1e9,
                          "dispatch": disp_bytes / (st["dispatch"] * 1e-3) / 1e9,
                          "combine": w.combine_bytes / (st["combine"] * 1e-3) / 1e9,
@@ -145,8 +212,41 @@ def main():
                                          "combine": w.combine_bytes / (st["combine"] * 1e-3) / 1e9 / PEAK_HBM_GBPS}},
         "stage_ms": st,
     }
-    if not args.no_cpu_baseline:
+    if args.staged:
+        result["staged"] = staged_run(w, blk, x, max(2, args.steps // 2))
+    if with_cpu:
         result["cpu_baseline"] = cpu_baseline(w, blk, min(args.cpu_sample, w.n))
+    del blk, x
+    torch.cuda.empty_cache()
+    return result
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="deepseek_v3_w8a16")
+    ap.add_argument("--all-workloads", action="store_true", help="one JSON line holding every synthetic workload")
+    ap.add_argument("--tokens", type=int, default=0, help="override the token count (parity/debug only)")
+    ap.add_argument("--materialize", action="store_true", help="gather rows into a sorted copy instead of "
+                    "reading them through the row map inside the GEMM")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--staged", action="store_true", help="also time the block with weights staged from pinned host memory")
+    ap.add_argument("--cpu-sample", type=int, default=128)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); use --gpus 1")
+
+    import torch
+    from moe_gen_amd import synthetic
+    torch.cuda.set_device(0)
+    if args.all_workloads:
+        result = run_workload("deepseek_v3_w8a16", args, not args.no_cpu_baseline)
+        result["workloads"] = [run_workload(n, args, not args.no_cpu_baseline)
+                               for n in synthetic.WORKLOADS if n != "deepseek_v3_w8a16"]
+    else:
+        result = run_workload(args.workload, args, not args.no_cpu_baseline)
     print(json.dumps(result))
 
 

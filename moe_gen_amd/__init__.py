@@ -5,4 +5,4 @@ from .config import DeepseekV2Config, DeepseekV3Config, MixtralConfig  # noqa: F
 from .deepseek_v2 import DeepseekV2MLP, DeepseekV2MoE  # noqa: F401
 from .deepseek_v3 import DeepseekV3MLP, DeepseekV3MoE, MoEGate  # noqa: F401
 from .mixtral import MixtralBlockSparseTop2MLP, MixtralSparseMoeBlock  # noqa: F401
-from .stager import Stager  # noqa: F401
+from .stager import StagedExpert, Stager  # noqa: F401

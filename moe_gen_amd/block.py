@@ -154,9 +154,11 @@ def collect_pointers(experts, cache):
     if engine_backed:
         cols = [[] for _ in range(6)]
         keys = []
+        # every expert of the layer is fetched below, so none of this layer's slots can be left
+        # behind by a skipped expert; one call reclaims what the previous layer left
+        if getattr(first, "expert_idx", -1) != -1:
+            first.core_engine.clear_expert_buffer(first.layer_idx, 0)
         for ex in experts:
-            if getattr(ex, "expert_idx", -1) != -1:
-                ex.core_engine.clear_expert_buffer(ex.layer_idx, ex.expert_idx)
             fetched = ex.core_engine.get_weights(ex.expert_weights_idx)
             keys.append((ex.core_engine, ex.expert_weights_idx))
             for c, t in zip(cols, _tensors_of(ex, fetched)):

@@ -168,8 +168,25 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     const int e = uni(lo);
     const int pe = uni(s_pref[e]);
     const int mt_e = uni(s_pref[e + 1]) - pe;
+    // Inside an expert, tiles are visited in groups of about GM consecutive M tiles (the expert's
+    // M tiles split as evenly as possible); within a group the M tile varies fastest.  The ~32
+    // workgroups an XCD runs at once then cover ~GM M tiles x a few N tiles, so each A panel and
+    // each B panel they touch is shared through the XCD's L2 (an expert with hundreds of M tiles
+    // would otherwise re-read A once per N tile, one with GM+1 would re-read B for the odd tile).
+    constexpr int GM = 8;
     const int local = v - pe * g.n_tiles_n;
-    const int n_tile = local / mt_e, m_tile = local - n_tile * mt_e;
+    const int ng = max(1, (mt_e + GM / 2) / GM);
+    const int base = mt_e / ng, extra = mt_e - base * ng;      // `extra` groups hold base+1 tiles
+    const int big = (base + 1) * g.n_tiles_n, cut = extra * big;
+    int gm, m0, rem;
+    if (local < cut) {
+        const int gi = local / big;
+        rem = local - gi * big; gm = base + 1; m0 = gi * (base + 1);
+    } else {
+        const int l2 = local - cut, sz = base * g.n_tiles_n, gi = l2 / sz;
+        rem = l2 - gi * sz; gm = base; m0 = extra * (base + 1) + gi * base;
+    }
+    const int n_tile = rem / gm, m_tile = m0 + (rem - n_tile * gm);
     const int row0 = uni(g.offsets[e]) + m_tile * BM;
     const int row_end = uni(g.offsets[e + 1]);
     const int n0 = n_tile * NBLK;

@@ -21,6 +21,23 @@ def _nbytes(shape, dtype) -> int:
     return n * torch.empty((), dtype=dtype).element_size()
 
 
+class StagedExpert(torch.nn.Module):
+    """An expert whose weights live in pinned host memory and reach the GPU through a Stager (or
+    MoE-Gen's core_engine): the attribute surface of the reference's Expert_Wrapper
+    (Wrapper.py:437-468) that block.collect_pointers consumes -- `.module`, `.core_engine`,
+    `.get_weights`, `.expert_weights_idx`, `.layer_idx`, `.expert_idx`, `.weight_dequant_scale`."""
+
+    def __init__(self, expert_module, layer_idx: int, expert_idx: int, core_engine, weight_dequant_scale=None):
+        super().__init__()
+        self.module = expert_module
+        self.layer_idx, self.expert_idx = layer_idx, expert_idx
+        self.core_engine = core_engine
+        self.get_weights = True
+        self.weight_dequant_scale = weight_dequant_scale
+        self.expert_weights_idx = (f"routed_expert_{layer_idx}_{expert_idx}" if expert_idx >= 0
+                                   else f"shared_expert_{layer_idx}")
+
+
 class Stager:
     """module_shapes: {module_type: {tensor_name: (shape, dtype)}} -- the reference's
     GPU_Buffer_Config.module_shapes (deepseekv3_initializer.py:938-957);
