@@ -290,28 +290,40 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
 #pragma unroll
         for (int j = 0; j < NJ; ++j) acc[mi][j] = f32x16{0};
 
-    // Operand fragments are double-buffered in registers: the 16-byte LDS reads of k-step s+1
-    // are issued before the MFMAs of k-step s.
-    auto compute = [&](const uint8_t* As) {
+    // Operand fragments are double-buffered in registers: the 16-byte LDS reads of k-step s+1 are
+    // issued before the MFMAs of k-step s.  The pipeline is rotated across the workgroup barrier:
+    // the MFMAs of the LAST k-step of a tile (whose fragments are already in registers) are issued
+    // after the barrier, behind the first LDS reads of the next tile, so the matrix core has work
+    // while those reads are in flight.
+    bf16x8 tf[2][MT], wf[2][NJ];
+    constexpr int NS = BK / 16, LAST = NS - 1;
+    auto read_frags = [&](const uint8_t* As, int s) {
         const uint8_t* Bs = As + A_STAGE;
-        bf16x8 tf[2][MT], wf[2][NJ];
-        auto read_frags = [&](int s, int buf) {
-            const uint32_t coff = (uint32_t)(((2 * s + fhalf) ^ fkey) << 4);
+        const uint32_t coff = (uint32_t)(((2 * s + fhalf) ^ fkey) << 4);
 #pragma unroll
-            for (int mi = 0; mi < MT; ++mi) tf[buf][mi] = *reinterpret_cast<const bf16x8*>(As + tok_off[mi] + coff);
+        for (int mi = 0; mi < MT; ++mi) tf[s & 1][mi] = *reinterpret_cast<const bf16x8*>(As + tok_off[mi] + coff);
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) wf[buf][j] = *reinterpret_cast<const bf16x8*>(Bs + w_off[j] + coff);
-        };
-        read_frags(0, 0);
+        for (int j = 0; j < NJ; ++j) wf[s & 1][j] = *reinterpret_cast<const bf16x8*>(Bs + w_off[j] + coff);
+    };
+    auto mfmas = [&](int s) {
 #pragma unroll
-        for (int s = 0; s < BK / 16; ++s) {
-            if (s + 1 < BK / 16) read_frags(s + 1, (s + 1) & 1);
+        for (int mi = 0; mi < MT; ++mi)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+                acc[mi][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[s & 1][j], tf[s & 1][mi], acc[mi][j], 0, 0, 0);
+    };
+    // multiplies k-steps 0 .. LAST-1 of the tile in `As`, preceded by the pending last k-step of the
+    // previous tile; leaves the fragments of k-step LAST in registers
+    auto compute = [&](const uint8_t* As, bool have_pending) {
+        read_frags(As, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (have_pending) mfmas(LAST);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < LAST; ++s) {
+            read_frags(As, s + 1);
             __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int mi = 0; mi < MT; ++mi)
-#pragma unroll
-                for (int j = 0; j < NJ; ++j)
-                    acc[mi][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[s & 1][j], tf[s & 1][mi], acc[mi][j], 0, 0, 0);
+            mfmas(s);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -325,15 +337,14 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     lds_store(smem0);
     if (nk > 1) gload(1);
     __syncthreads();
-    int kt = 0;
     const bool mfma_first = wave < 4;   // waves w and w+4 share a SIMD
-    for (; kt < nk; ++kt) {
+    for (int kt = 0; kt < nk; ++kt) {
         const uint8_t* rd = (kt & 1) ? smem1 : smem0;
         uint8_t* wr = (kt & 1) ? smem0 : smem1;
         // the wave that is multiplying outranks its SIMD partner that is moving data
         if (mfma_first) {
             __builtin_amdgcn_s_setprio(2);
-            compute(rd);
+            compute(rd, kt > 0);
             __builtin_amdgcn_s_setprio(0);
             if (kt + 1 < nk) lds_store(wr);
             if (kt + 2 < nk) gload(kt + 2);
@@ -341,11 +352,12 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
             if (kt + 1 < nk) lds_store(wr);
             if (kt + 2 < nk) gload(kt + 2);
             __builtin_amdgcn_s_setprio(2);
-            compute(rd);
+            compute(rd, kt > 0);
             __builtin_amdgcn_s_setprio(0);
         }
-        __syncthreads();
+        __syncthreads();   // (waits for this wave's LDS reads and writes, then for the other waves)
     }
+    mfmas(LAST);
 
     // ---- epilogue ----
     // acc[mi][j][i]: token row = 32*mi + lane%32 of the wave's M range; output column
