@@ -51,3 +51,97 @@ def test_stager_overlaps_with_compute():
         assert torch.isfinite(s) and same
     torch.cuda.synchronize()
     st.close()
+
+
+class FakeCoreEngine:
+    """Stands in for MoE-Gen's pybind `core_engine` (MoE_Gen_Binding.cpp:45-65): hands out device
+    tensors by module key and records the protocol calls."""
+
+    def __init__(self, weights):
+        self.weights, self.calls, self.held = weights, [], set()
+
+    def get_weights(self, key):
+        self.calls.append(("get", key)); self.held.add(key)
+        return self.weights[key]
+
+    def free_weights_buffer(self, key):
+        self.calls.append(("free", key)); self.held.remove(key)
+
+    def clear_expert_buffer(self, layer_idx, expert_idx):
+        self.calls.append(("clear", layer_idx, expert_idx))
+
+
+class ExpertWrapperLike(torch.nn.Module):
+    """Attribute-for-attribute what the reference's Expert_Wrapper exposes (Wrapper.py:437-468)."""
+
+    def __init__(self, module, layer_idx, expert_idx, core_engine, scales):
+        super().__init__()
+        self.module, self.layer_idx, self.expert_idx = module, layer_idx, expert_idx
+        self.core_engine, self.get_weights, self.weight_dequant_scale = core_engine, True, scales
+        self.expert_weights_idx = (f"routed_expert_{layer_idx}_{expert_idx}" if expert_idx >= 0
+                                   else f"shared_expert_{layer_idx}")
+
+
+@pytest.mark.parametrize("name", ["deepseek_v3_w8a16", "deepseek_v2_236b"])
+def test_block_with_engine_backed_experts(name):
+    """The block fed through MoE-Gen's expert-wrapper protocol gives the same bits as with resident
+    weights, and calls get_weights / free_weights_buffer once per expert."""
+    from moe_gen_amd import synthetic
+    w = synthetic.WORKLOADS[name].scaled(n=256, h=512, I=256, seq=64)
+    blk = synthetic.build_block(w, device="cuda", gen_device="cpu")
+    x = synthetic.hidden_states(w, "cpu").cuda()
+    ref = blk(x).clone()
+    names = blk.experts[0].names
+    L = 7
+    weights, wrapped = {}, []
+
+    def detach(mlp, key):
+        weights[key] = {f"{n}.weight": getattr(mlp, n).weight.data.clone() for n in names}
+        scales = {f"{n}.weight_scale_inv": getattr(mlp, n).weight_scale_inv.data for n in names} if w.fp8 else None
+        for n in names:                                   # placeholders, as MoE-Gen leaves them
+            getattr(mlp, n).weight.data = torch.zeros(1, dtype=torch.bfloat16, device="cuda")
+        return scales
+
+    eng = FakeCoreEngine(weights)
+    for e, ex in enumerate(blk.experts):
+        wrapped.append(ExpertWrapperLike(ex, L, e, eng, detach(ex, f"routed_expert_{L}_{e}")))
+    blk.experts = torch.nn.ModuleList(wrapped)
+    blk.shared_experts = ExpertWrapperLike(blk.shared_experts, L, -1, eng, detach(blk.shared_experts, f"shared_expert_{L}"))
+    out = blk(x)
+    torch.cuda.synchronize()
+    assert torch.equal(out, ref)
+    gets = [c[1] for c in eng.calls if c[0] == "get"]
+    frees = [c[1] for c in eng.calls if c[0] == "free"]
+    assert sorted(gets) == sorted(frees) == sorted(weights) and not eng.held
+    assert ("clear", L, 0) in eng.calls
+
+
+def test_block_with_library_stager():
+    """Same, with the library's own Stager delivering fp8 experts from pinned host memory."""
+    from moe_gen_amd import StagedExpert, Stager, synthetic
+    w = synthetic.WORKLOADS["deepseek_v3_w8a16"].scaled(n=256, h=512, I=256, E=16, n_group=4, topk_group=2, k=4, seq=64)
+    blk = synthetic.build_block(w, device="cuda", gen_device="cpu")
+    x = synthetic.hidden_states(w, "cpu").cuda()
+    ref = blk(x).clone()
+    names = blk.experts[0].names
+    fp8 = torch.float8_e4m3fn
+    shapes = {"routed_expert": {f"{n}.weight": (tuple(getattr(blk.experts[0], n).weight.shape), fp8) for n in names},
+              "shared_expert": {f"{n}.weight": (tuple(getattr(blk.shared_experts, n).weight.shape), fp8) for n in names}}
+    st = Stager(shapes, {"routed_expert": w.E, "shared_expert": 1}, model_type="deepseek_v3", num_hidden_layers=8,
+                num_local_experts=w.E)
+    L = 5
+    wrapped = []
+    for e, ex in enumerate(blk.experts):
+        st.add_module(f"routed_expert_{L}_{e}", "routed_expert",
+                      {f"{n}.weight": getattr(ex, n).weight.data.cpu().pin_memory() for n in names})
+        wrapped.append(StagedExpert(ex, L, e, st, {f"{n}.weight_scale_inv": getattr(ex, n).weight_scale_inv.data for n in names}))
+    sh = blk.shared_experts
+    st.add_module(f"shared_expert_{L}", "shared_expert", {f"{n}.weight": getattr(sh, n).weight.data.cpu().pin_memory() for n in names})
+    blk.experts = torch.nn.ModuleList(wrapped)
+    blk.shared_experts = StagedExpert(sh, L, -1, st, {f"{n}.weight_scale_inv": getattr(sh, n).weight_scale_inv.data for n in names})
+    for _ in range(3):                                    # slots are recycled between calls
+        out = blk(x)
+    torch.cuda.synchronize()
+    assert torch.equal(out, ref)
+    assert st.stats()[0] >= 3 * (w.E + 1)
+    st.close()
