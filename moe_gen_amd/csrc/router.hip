@@ -11,7 +11,9 @@
 // exactly that order at twice the rate of the vector ALU: v_mfma_f32_32x32x1_2b_f32
 // performs one rank-1 update D = a * b^T + C per instruction, i.e. a single fused
 // multiply-add per output element per k.  Operands are staged through LDS as fp32
-// (bf16 -> fp32 is a 16-bit shift, exact).
+// (bf16 -> fp32 is a 16-bit shift, exact).  For E <= 16 the 4x4x1 form of the same
+// instruction is used (16 blocks of 4 tokens x 4 experts, 8 cycles): no padding to 32
+// experts and an 8x shorter dependency chain per k.
 //
 // Selection.  After the K loop the block's logits sit in LDS; each wave then
 // routes one token at a time with the 64 lanes strided over the experts
@@ -24,19 +26,19 @@
 namespace moe {
 namespace {
 
-constexpr int KC = 32;           // k elements per LDS stage
-constexpr int LDK = KC + 4;      // padded fp32 row stride (144 B): conflict-free b128 reads
-constexpr int MAX_EJ = 4;        // experts per lane (E <= 256)
-
+// Lanes of a wave work in groups of GW (64, or 16 when E <= 16): a group routes one token, its
+// lanes strided over the experts (lane g of the group holds experts g, g+GW, ...).  Reductions are
+// xor butterflies inside the group, so every lane of the group ends with the same value.
 struct ArgMax {
     float v;
     int i;
 };
 
-// max by value, equal values -> lower index; all lanes receive the result
-__device__ __forceinline__ ArgMax wave_argmax(ArgMax a) {
+// max by value, equal values -> lower index
+template <int GW>
+__device__ __forceinline__ ArgMax group_argmax(ArgMax a) {
 #pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) {
+    for (int m = GW / 2; m >= 1; m >>= 1) {
         float ov = __shfl_xor(a.v, m);
         int oi = __shfl_xor(a.i, m);
         bool take = (ov > a.v) || (ov == a.v && oi < a.i);
@@ -46,38 +48,44 @@ __device__ __forceinline__ ArgMax wave_argmax(ArgMax a) {
     return a;
 }
 
-__device__ __forceinline__ float wave_max(float v) {
+template <int GW>
+__device__ __forceinline__ float group_max(float v) {
 #pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m));
+    for (int m = GW / 2; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m));
     return v;
 }
 
-// butterfly 32,16,8,4,2,1: p[l] = p[l] + p[l^m]; fp32 addition commutes, so every
-// lane ends with the same value
-__device__ __forceinline__ float wave_sum_butterfly(float v) {
+// The canonical sum over experts: 64 strided partials folded by the butterfly 32,16,8,4,2,1
+// (p[l] += p[l^m]; fp32 addition commutes).  With E <= 16 the partials of lanes 16..63 are +0, the
+// steps 32 and 16 add +0 to non-negative values, and the remaining steps are the 16-lane butterfly.
+template <int GW>
+__device__ __forceinline__ float group_sum_butterfly(float v) {
 #pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v = v + __shfl_xor(v, m);
+    for (int m = GW / 2; m >= 1; m >>= 1) v = v + __shfl_xor(v, m);
     return v;
 }
 
 constexpr float kNegInf = -__builtin_inff();
 constexpr int kBigIdx = 0x7fffffff;
 
-// Routes one token whose logits are in `row` (LDS, E valid entries).
-__device__ void route_token(const float* row, const float* __restrict__ bias,
-                            const moe_router_params& p, int32_t* __restrict__ idx_out,
-                            float* __restrict__ w_out, float* __restrict__ logits_out) {
-    const int lane = threadIdx.x & 63;
+// Routes one token per lane group; `row` points at the group's logits (LDS, E valid entries).
+// `live` is false for groups without a token (they run the same code on a valid row, store nothing).
+template <int GW>
+__device__ void route_token(const float* row, const float* __restrict__ bias, const moe_router_params& p,
+                            int32_t* __restrict__ idx_out, float* __restrict__ w_out,
+                            float* __restrict__ logits_out, bool live) {
+    constexpr int MAX_EJ = GW == 64 ? 4 : 1;   // experts per lane (E <= 256, or E <= 16)
+    const int lane = threadIdx.x & 63, gl = lane & (GW - 1), gbase = lane - gl;
     const int E = p.n_experts;
     float L[MAX_EJ], s[MAX_EJ], c[MAX_EJ];
     bool valid[MAX_EJ];
 #pragma unroll
     for (int j = 0; j < MAX_EJ; ++j) {
-        int e = lane + 64 * j;
+        int e = gl + GW * j;
         valid[j] = e < E;
         L[j] = valid[j] ? row[e] : 0.0f;
         if (p.logits_bf16) L[j] = round_to_bf16(L[j]);
-        if (logits_out && valid[j]) logits_out[e] = L[j];
+        if (logits_out && valid[j] && live) logits_out[e] = L[j];
     }
     if (p.scoring == MOE_SCORE_SIGMOID) {
 #pragma unroll
@@ -86,21 +94,21 @@ __device__ void route_token(const float* row, const float* __restrict__ bias,
         float m = kNegInf;
 #pragma unroll
         for (int j = 0; j < MAX_EJ; ++j) m = valid[j] ? fmaxf(m, L[j]) : m;
-        m = wave_max(m);
+        m = group_max<GW>(m);
         float part = 0.0f;
 #pragma unroll
         for (int j = 0; j < MAX_EJ; ++j) {
             s[j] = valid[j] ? canon_expf(L[j] - m) : 0.0f;
             part = part + s[j];  // adding +0 for absent experts changes nothing
         }
-        float sum = wave_sum_butterfly(part);
+        float sum = group_sum_butterfly<GW>(part);
 #pragma unroll
         for (int j = 0; j < MAX_EJ; ++j) s[j] = s[j] / sum;
     }
 #pragma unroll
     for (int j = 0; j < MAX_EJ; ++j) {
         c[j] = s[j];
-        if (p.method == MOE_TOPK_NOAUX_TC && bias != nullptr && valid[j]) c[j] = s[j] + bias[lane + 64 * j];
+        if (p.method == MOE_TOPK_NOAUX_TC && bias != nullptr && valid[j]) c[j] = s[j] + bias[gl + GW * j];
     }
 
     float tmp[MAX_EJ];
@@ -111,31 +119,31 @@ __device__ void route_token(const float* row, const float* __restrict__ bias,
         const int G = p.n_group, per = E / G;
         int grp[MAX_EJ];
 #pragma unroll
-        for (int j = 0; j < MAX_EJ; ++j) grp[j] = valid[j] ? (lane + 64 * j) / per : 0;
-        float my_gs = kNegInf;  // lane g keeps the score of group g
+        for (int j = 0; j < MAX_EJ; ++j) grp[j] = valid[j] ? (gl + GW * j) / per : 0;
+        float my_gs = kNegInf;  // lane g of the group keeps the score of expert-group g
         for (int g = 0; g < G; ++g) {
             ArgMax a{kNegInf, kBigIdx};
 #pragma unroll
             for (int j = 0; j < MAX_EJ; ++j)
-                if (valid[j] && grp[j] == g && (c[j] > a.v || a.i == kBigIdx)) a = ArgMax{c[j], lane + 64 * j};
-            a = wave_argmax(a);
+                if (valid[j] && grp[j] == g && (c[j] > a.v || a.i == kBigIdx)) a = ArgMax{c[j], gl + GW * j};
+            a = group_argmax<GW>(a);
             float gs = a.v;
             if (p.method == MOE_TOPK_NOAUX_TC) {  // sum of the two largest of the group
                 float v2 = kNegInf;
 #pragma unroll
                 for (int j = 0; j < MAX_EJ; ++j)
-                    if (valid[j] && grp[j] == g && (lane + 64 * j) != a.i) v2 = fmaxf(v2, c[j]);
-                v2 = wave_max(v2);
+                    if (valid[j] && grp[j] == g && (gl + GW * j) != a.i) v2 = fmaxf(v2, c[j]);
+                v2 = group_max<GW>(v2);
                 gs = a.v + v2;
             }
-            if (lane == g) my_gs = gs;
+            if (gl == g) my_gs = gs;
         }
         uint32_t keep = 0;
         bool gtaken = false;
         for (int r = 0; r < p.topk_group; ++r) {
-            ArgMax a = (lane < G && !gtaken) ? ArgMax{my_gs, lane} : ArgMax{kNegInf, kBigIdx};
-            a = wave_argmax(a);
-            if (lane == a.i) gtaken = true;
+            ArgMax a = (gl < G && !gtaken) ? ArgMax{my_gs, gl} : ArgMax{kNegInf, kBigIdx};
+            a = group_argmax<GW>(a);
+            if (gl == a.i) gtaken = true;
             keep |= 1u << a.i;
         }
 #pragma unroll
@@ -143,34 +151,36 @@ __device__ void route_token(const float* row, const float* __restrict__ bias,
             tmp[j] = (valid[j] && ((keep >> grp[j]) & 1u)) ? c[j] : 0.0f;  // masked_fill(~mask, 0.0)
     }
 
-    // top-k by repeated argmax; lane r keeps slot r
-    bool taken[MAX_EJ] = {false, false, false, false};
+    // top-k by repeated argmax; lane r of the group keeps slot r
+    bool taken[MAX_EJ];
+#pragma unroll
+    for (int j = 0; j < MAX_EJ; ++j) taken[j] = false;
     int my_idx = 0;
     float my_w = 0.0f;
     for (int r = 0; r < p.top_k; ++r) {
         ArgMax a{kNegInf, kBigIdx};
 #pragma unroll
         for (int j = 0; j < MAX_EJ; ++j)
-            if (valid[j] && !taken[j] && (a.i == kBigIdx || tmp[j] > a.v)) a = ArgMax{tmp[j], lane + 64 * j};
-        a = wave_argmax(a);
-        const int owner = a.i & 63, oj = a.i >> 6;
+            if (valid[j] && !taken[j] && (a.i == kBigIdx || tmp[j] > a.v)) a = ArgMax{tmp[j], gl + GW * j};
+        a = group_argmax<GW>(a);
+        const int owner = a.i & (GW - 1), oj = a.i / GW;
         float sv = 0.0f;
 #pragma unroll
         for (int j = 0; j < MAX_EJ; ++j) {
-            if (lane == owner && oj == j) taken[j] = true;
+            if (gl == owner && oj == j) taken[j] = true;
             if (oj == j) sv = s[j];
         }
-        sv = __shfl(sv, owner);
+        sv = __shfl(sv, gbase + owner);
         // V3 gathers the unbiased score; V2 / Mixtral keep the selected value
         float wv = (p.method == MOE_TOPK_NOAUX_TC) ? sv : a.v;
-        if (lane == r) {
+        if (gl == r) {
             my_idx = a.i;
             my_w = wv;
         }
     }
     if (p.top_k > 1 && p.norm_topk_prob) {
         float sum = 0.0f;
-        for (int r = 0; r < p.top_k; ++r) sum = sum + __shfl(my_w, r);
+        for (int r = 0; r < p.top_k; ++r) sum = sum + __shfl(my_w, gbase + r);
         float den = sum + p.norm_eps;
         my_w = my_w / den;
         if (p.scale_mode == MOE_SCALE_ALWAYS) my_w = my_w * p.routed_scaling_factor;
@@ -178,21 +188,31 @@ __device__ void route_token(const float* row, const float* __restrict__ bias,
         my_w = my_w * p.routed_scaling_factor;
     }
     if (p.weights_bf16) my_w = round_to_bf16(my_w);
-    if (lane < p.top_k) {
-        idx_out[lane] = my_idx;
-        w_out[lane] = my_w;
+    if (live && gl < p.top_k) {
+        idx_out[gl] = my_idx;
+        w_out[gl] = my_w;
     }
 }
 
-// NEB: 32-expert MFMA blocks per wave (1 or 2); WE / WT: waves along experts / tokens.
-template <int NEB, int WE, int WT>
+// Two logit engines share the kernel:
+//  SMALL == false: v_mfma_f32_32x32x1_2b_f32.  NEB: 32-expert MFMA blocks per wave (1 or 2);
+//                  WE / WT: waves along experts / tokens.
+//  SMALL == true : v_mfma_f32_4x4x1_16b_f32 for E <= 16 (Mixtral's 8 experts): one instruction is
+//                  64 tokens x 4 experts in 8 cycles, so nothing is padded to 32 experts and the
+//                  sequential-in-k dependency chain is 8x shorter.  NEB = groups of 4 experts (1..4),
+//                  WE = 1.
+// Global loads run two k-stages ahead in registers (two register sets, loop unrolled by two), which
+// is what hides the load latency when only a few workgroups exist (small token counts).
+template <bool SMALL, int NEB, int WE, int WT>
 __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ wg, const float* __restrict__ bias,
     moe_router_params p, int32_t* __restrict__ topk_idx, float* __restrict__ topk_w,
     float* __restrict__ logits_out) {
+    constexpr int KC = SMALL ? 64 : 32;  // k elements per LDS stage
+    constexpr int LDK = KC + 4;          // padded fp32 row stride: conflict-free 16-byte reads
     constexpr int NT = 64 * WE * WT;  // threads
     constexpr int BT = 64 * WT;       // tokens per block
-    constexpr int EP = 32 * NEB * WE; // padded experts per block
+    constexpr int EP = SMALL ? 4 * NEB : 32 * NEB * WE;  // padded experts per block
     constexpr int XCH = BT * (KC / 8), WCH = EP * (KC / 8);  // 16-byte chunks per stage
     constexpr int XPT = (XCH + NT - 1) / NT, WPT = (WCH + NT - 1) / NT;
     constexpr int TILE_F = (BT + EP) * LDK, LOGIT_F = BT * EP;
@@ -206,25 +226,25 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     const int n = p.n_tokens, h = p.hidden, E = p.n_experts;
     const int t0 = blockIdx.x * BT;
 
-    u32x4 xr[XPT], wr[WPT];
-    auto load_stage = [&](int k0) {
+    u32x4 xr[2][XPT], wr[2][WPT];
+    auto load_stage = [&](int k0, int set) {
 #pragma unroll
         for (int i = 0; i < XPT; ++i) {
             int c = tid + i * NT;
-            int row = c >> 2, kk = k0 + (c & 3) * 8;
+            int row = c / (KC / 8), kk = k0 + (c % (KC / 8)) * 8;
             int t = min(t0 + row, n - 1);
-            xr[i] = (c < XCH && kk < h) ? *reinterpret_cast<const u32x4*>(x + (size_t)t * h + kk) : u32x4{0, 0, 0, 0};
+            xr[set][i] = (c < XCH && kk < h) ? *reinterpret_cast<const u32x4*>(x + (size_t)t * h + kk) : u32x4{0, 0, 0, 0};
         }
 #pragma unroll
         for (int i = 0; i < WPT; ++i) {
             int c = tid + i * NT;
-            int row = c >> 2, kk = k0 + (c & 3) * 8;
+            int row = c / (KC / 8), kk = k0 + (c % (KC / 8)) * 8;
             int e = min(row, E - 1);
-            wr[i] = (c < WCH && kk < h) ? *reinterpret_cast<const u32x4*>(wg + (size_t)e * h + kk) : u32x4{0, 0, 0, 0};
+            wr[set][i] = (c < WCH && kk < h) ? *reinterpret_cast<const u32x4*>(wg + (size_t)e * h + kk) : u32x4{0, 0, 0, 0};
         }
     };
     auto store_chunk = [&](float* base, int c, u32x4 v) {
-        float* d = base + (c >> 2) * LDK + (c & 3) * 8;
+        float* d = base + (c / (KC / 8)) * LDK + (c % (KC / 8)) * 8;
         f32x4 lo, hi;
         lo[0] = __uint_as_float(v[0] << 16); lo[1] = __uint_as_float(v[0] & 0xffff0000u);
         lo[2] = __uint_as_float(v[1] << 16); lo[3] = __uint_as_float(v[1] & 0xffff0000u);
@@ -233,81 +253,128 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
         *reinterpret_cast<f32x4*>(d) = lo;
         *reinterpret_cast<f32x4*>(d + 4) = hi;
     };
-    auto store_stage = [&]() {
+    auto store_stage = [&](int set) {
 #pragma unroll
         for (int i = 0; i < XPT; ++i) {
             int c = tid + i * NT;
-            if (c < XCH) store_chunk(Xs, c, xr[i]);
+            if (c < XCH) store_chunk(Xs, c, xr[set][i]);
         }
 #pragma unroll
         for (int i = 0; i < WPT; ++i) {
             int c = tid + i * NT;
-            if (c < WCH) store_chunk(Ws, c, wr[i]);
+            if (c < WCH) store_chunk(Ws, c, wr[set][i]);
         }
     };
 
-    f32x32 acc0 = {0}, acc1 = {0};
+    f32x32 acc0 = {0}, acc1 = {0};          // SMALL == false
+    f32x4 acc4[SMALL ? NEB : 1];            // SMALL == true: group j = experts 4j .. 4j+3
+#pragma unroll
+    for (int j = 0; j < (SMALL ? NEB : 1); ++j) acc4[j] = f32x4{0, 0, 0, 0};
     const float* a_row = Xs + (wt * 64 + lane) * LDK;
-    const float* b0_row = Ws + (NEB == 2 ? (we * 64 + lane) : (we * 32 + (lane & 31))) * LDK;
-    const float* b1_row = Ws + (we * 64 + (lane ^ 32)) * LDK;  // only read when NEB == 2
+    const float* b0_row = SMALL ? Ws + (lane & 3) * LDK
+                                : Ws + (NEB == 2 ? (we * 64 + lane) : (we * 32 + (lane & 31))) * LDK;
+    const float* b1_row = Ws + (we * 64 + (lane ^ 32)) * LDK;  // only read when !SMALL && NEB == 2
 
-    const int nstage = (h + KC - 1) / KC;
-    load_stage(0);
-    for (int st = 0; st < nstage; ++st) {
-        store_stage();
-        __syncthreads();
-        if (st + 1 < nstage) load_stage((st + 1) * KC);
+    // operands of k..k+3 are read (16 bytes per lane) one step ahead of the MFMAs that use them
+    constexpr int NB4 = SMALL ? NEB : 2;
+    auto read_ops = [&](int k4, f32x4& a, f32x4 (&b)[NB4]) {
+        a = *reinterpret_cast<const f32x4*>(a_row + k4 * 4);
+        if (SMALL) {
+#pragma unroll
+            for (int j = 0; j < NEB; ++j) b[j] = *reinterpret_cast<const f32x4*>(b0_row + j * 4 * LDK + k4 * 4);
+        } else {
+            b[0] = *reinterpret_cast<const f32x4*>(b0_row + k4 * 4);
+            if (NEB == 2) b[1] = *reinterpret_cast<const f32x4*>(b1_row + k4 * 4);
+        }
+    };
+    auto multiply_stage = [&]() {
+        f32x4 a[2], b[2][NB4];
+        read_ops(0, a[0], b[0]);
 #pragma unroll
         for (int k4 = 0; k4 < KC / 4; ++k4) {
-            f32x4 a = *reinterpret_cast<const f32x4*>(a_row + k4 * 4);
-            f32x4 b0 = *reinterpret_cast<const f32x4*>(b0_row + k4 * 4);
-            f32x4 b1;
-            if (NEB == 2) b1 = *reinterpret_cast<const f32x4*>(b1_row + k4 * 4);
+            if (k4 + 1 < KC / 4) read_ops(k4 + 1, a[(k4 + 1) & 1], b[(k4 + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
-                acc0 = __builtin_amdgcn_mfma_f32_32x32x1f32(a[kk], b0[kk], acc0, 0, 0, 0);
-                if (NEB == 2) acc1 = __builtin_amdgcn_mfma_f32_32x32x1f32(a[kk], b1[kk], acc1, 0, 0, 0);
+                if (SMALL) {
+#pragma unroll
+                    for (int j = 0; j < NEB; ++j)
+                        acc4[j] = __builtin_amdgcn_mfma_f32_4x4x1f32(a[k4 & 1][kk], b[k4 & 1][j][kk], acc4[j], 0, 0, 0);
+                } else {
+                    acc0 = __builtin_amdgcn_mfma_f32_32x32x1f32(a[k4 & 1][kk], b[k4 & 1][0][kk], acc0, 0, 0, 0);
+                    if (NEB == 2) acc1 = __builtin_amdgcn_mfma_f32_32x32x1f32(a[k4 & 1][kk], b[k4 & 1][1][kk], acc1, 0, 0, 0);
+                }
             }
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __syncthreads();
-    }
+    };
 
-    // accumulators -> LDS logits[token][expert].  In block b of the 2-block MFMA
-    // result, register 16*b+i of lane l is row 8*(i/4) + 4*(l/32) + i%4, column l%32.
+    const int nstage = (h + KC - 1) / KC;
+    load_stage(0, 0);
+    if (nstage > 1) load_stage(KC, 1);
+    auto stage = [&](int st, int set) {      // set == st & 1, a literal at both call sites
+        store_stage(set);
+        __syncthreads();
+        if (st + 2 < nstage) load_stage((st + 2) * KC, set);
+        multiply_stage();
+        __syncthreads();
+    };
+    int st = 0;
+    for (; st + 1 < nstage; st += 2) {
+        stage(st, 0);
+        stage(st + 1, 1);
+    }
+    if (st < nstage) stage(st, 0);
+
+    // accumulators -> LDS logits[token][expert]
     float* lg = lds;
+    if (SMALL) {
+        // register i of lane l of group j: token 4*(l/4) + i, expert 4*j + l%4
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
+        for (int j = 0; j < NEB; ++j)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            int tl = wt * 64 + 32 * b + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
-            if (NEB == 2) {
-                int e0 = we * 64 + 32 * b + (lane & 31);        // acc0: A block b x B0 block b
-                int e1 = we * 64 + 32 * (1 - b) + (lane & 31);  // acc1: A block b x B1 block b
-                lg[tl * EP + e0] = acc0[16 * b + i];
-                lg[tl * EP + e1] = acc1[16 * b + i];
-            } else {
-                lg[tl * EP + we * 32 + (lane & 31)] = acc0[16 * b + i];
+            for (int i = 0; i < 4; ++i) lg[(wt * 64 + 4 * (lane >> 2) + i) * EP + 4 * j + (lane & 3)] = acc4[j][i];
+    } else {
+        // in block b of the 2-block MFMA result, register 16*b+i of lane l is row
+        // 8*(i/4) + 4*(l/32) + i%4, column l%32
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                int tl = wt * 64 + 32 * b + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
+                if (NEB == 2) {
+                    int e0 = we * 64 + 32 * b + (lane & 31);        // acc0: A block b x B0 block b
+                    int e1 = we * 64 + 32 * (1 - b) + (lane & 31);  // acc1: A block b x B1 block b
+                    lg[tl * EP + e0] = acc0[16 * b + i];
+                    lg[tl * EP + e1] = acc1[16 * b + i];
+                } else {
+                    lg[tl * EP + we * 32 + (lane & 31)] = acc0[16 * b + i];
+                }
             }
         }
     }
     __syncthreads();
 
-    constexpr int NW = WE * WT;
-    for (int tl = wave; tl < BT; tl += NW) {
-        int t = t0 + tl;
-        if (t >= n) break;
-        route_token(lg + tl * EP, bias, p, topk_idx + (size_t)t * p.top_k, topk_w + (size_t)t * p.top_k,
-                    logits_out ? logits_out + (size_t)t * E : nullptr);
+    // selection: a lane group per token (4 tokens per wave at a time when E <= 16)
+    constexpr int NW = WE * WT, GW = SMALL ? 16 : 64, TPW = 64 / GW;
+    for (int tb = wave * TPW; tb < BT; tb += NW * TPW) {
+        if (t0 + tb >= n) break;
+        const int tl = tb + (lane / GW);
+        const int t = t0 + tl;
+        const bool live = t < n;
+        const int tr = live ? t : n - 1, tlr = live ? tl : tb;
+        route_token<GW>(lg + tlr * EP, bias, p, topk_idx + (size_t)tr * p.top_k, topk_w + (size_t)tr * p.top_k,
+                        logits_out ? logits_out + (size_t)tr * E : nullptr, live);
     }
 }
 
-template <int NEB, int WE, int WT>
+template <bool SMALL, int NEB, int WE, int WT>
 int launch(const void* x, const void* w, const float* bias, const moe_router_params& p, int32_t* idx,
            float* tw, float* lo, hipStream_t st) {
     constexpr int BT = 64 * WT;
     dim3 grid((p.n_tokens + BT - 1) / BT), block(64 * WE * WT);
-    hipLaunchKernelGGL((router_kernel<NEB, WE, WT>), grid, block, 0, st, (const uint16_t*)x, (const uint16_t*)w,
-                       bias, p, idx, tw, lo);
+    hipLaunchKernelGGL((router_kernel<SMALL, NEB, WE, WT>), grid, block, 0, st, (const uint16_t*)x,
+                       (const uint16_t*)w, bias, p, idx, tw, lo);
     MOE_HIP_CHECK(hipGetLastError());
     return MOE_OK;
 }
@@ -343,9 +410,15 @@ extern "C" int moe_router(const void* x, const void* w_gate, const float* bias, 
     }
     hipStream_t st = as_stream(stream);
     const int E = p.n_experts;
-    if (E <= 32) return launch<1, 1, 4>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    if (E <= 64) return launch<2, 1, 4>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    if (E <= 128) return launch<2, 2, 2>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    if (E <= 192) return launch<2, 3, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    return launch<2, 4, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    // few tokens: one wave per workgroup so that the (sequential-in-k) work spreads over more CUs
+    const bool few = p.n_tokens <= 64 * 256;
+    if (E <= 4) return launch<true, 1, 1, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    if (E <= 8) return launch<true, 2, 1, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    if (E <= 16) return launch<true, 4, 1, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    if (E <= 32) return few ? launch<false, 1, 1, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st)
+                            : launch<false, 1, 1, 4>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    if (E <= 64) return launch<false, 1, 2, 2>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    if (E <= 128) return launch<false, 2, 2, 2>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    if (E <= 192) return launch<false, 2, 3, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    return launch<false, 2, 4, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
 }
