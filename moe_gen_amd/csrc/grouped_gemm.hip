@@ -31,7 +31,7 @@
 //
 // The MFMA is issued with the WEIGHT fragment as srcA and the TOKEN fragment as srcB, so
 // a lane ends up holding 4 consecutive output columns of one token row per register
-// quad: the epilogue packs them into one 8-byte store.
+// quad; the epilogue transposes them through LDS into 16-byte-per-lane row-contiguous stores.
 
 #include "common.h"
 
@@ -361,46 +361,55 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
 
     // ---- epilogue ----
     // acc[mi][j][i]: token row = 32*mi + lane%32 of the wave's M range; output column
-    // = tile column base + 8*(i/4) + 4*(lane/32) + i%4.
-    const int rows_here = min(BM, row_end - row0);
+    // = tile column base + 8*(i/4) + 4*(lane/32) + i%4, i.e. a lane holds 4 consecutive columns
+    // (8 bytes) of one row per register quad.  Storing those directly would issue 8-byte writes to
+    // 32 different rows per instruction; instead each wave transposes its outputs through its own
+    // slice of the (now idle) LDS stages and writes 16 bytes per lane, whole 64/128-byte row
+    // segments per 4/8 lanes.  (All waves passed the loop's last barrier, so no one reads the stages.)
+    constexpr int CW = SWIGLU ? 16 * NJ : 32 * NJ;   // output columns of this wave
+    constexpr int RBW = CW * 2;                      // bytes per output row of this wave
+    constexpr int CPR = RBW / 16;                    // 16-byte chunks per row (4 or 8)
+    constexpr int KSH = CPR == 8 ? 0 : 1;            // swizzle key = (row >> KSH) & (CPR-1)
+    uint8_t* ep = ((wave < 4) ? smem0 : smem1) + (wave & 3) * (32 * MT * RBW);
 #pragma unroll
     for (int mi = 0; mi < MT; ++mi) {
-        const int ml = wm * 32 * MT + 32 * mi + frow;
-        if (ml >= rows_here) continue;
-        uint16_t* crow = g.c + (size_t)(row0 + ml) * N;
-        if (SWIGLU) {
+        const int r = 32 * mi + frow;
+        uint8_t* erow = ep + r * RBW + fhalf * 8;
+        const int key = (r >> KSH) & (CPR - 1);
 #pragma unroll
-            for (int j = 0; j < NJ / 2; ++j) {
+        for (int jj = 0; jj < (SWIGLU ? NJ / 2 : NJ); ++jj) {
 #pragma unroll
-                for (int qd = 0; qd < 4; ++qd) {
-                    const int n = n0 + wn * (16 * NJ) + 32 * j + 8 * qd + 4 * fhalf;
+            for (int qd = 0; qd < 4; ++qd) {
+                u32x2 pk;
+                if (SWIGLU) {
                     float o[4];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        float gv = bf16r(acc[mi][j][4 * qd + i]);
-                        float uv = bf16r(acc[mi][j + NJ / 2][4 * qd + i]);
+                        float gv = bf16r(acc[mi][jj][4 * qd + i]);
+                        float uv = bf16r(acc[mi][jj + NJ / 2][4 * qd + i]);
                         float sg = bf16r(gv * __builtin_amdgcn_rcpf(1.0f + __expf(-gv)));
                         o[i] = sg * uv;
                     }
-                    if (n < N) {
-                        u32x2 pk = {pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3])};
-                        *reinterpret_cast<u32x2*>(crow + n) = pk;
-                    }
+                    pk = u32x2{pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3])};
+                } else {
+                    pk = u32x2{pack_bf16(acc[mi][jj][4 * qd], acc[mi][jj][4 * qd + 1]),
+                               pack_bf16(acc[mi][jj][4 * qd + 2], acc[mi][jj][4 * qd + 3])};
                 }
+                *reinterpret_cast<u32x2*>(erow + (((4 * jj + qd) ^ key) << 4)) = pk;
             }
-        } else {
+        }
+    }
+    const int rows_here = min(BM, row_end - row0) - wm * 32 * MT;   // valid rows of this wave
+    const int ncol0 = n0 + wn * CW;
+    constexpr int RPP = 64 / CPR;                    // rows per pass
+    const int rr = lane / CPR, cc = lane % CPR;
+    if (ncol0 + cc * 8 < N) {
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-#pragma unroll
-                for (int qd = 0; qd < 4; ++qd) {
-                    const int n = n0 + wn * (32 * NJ) + 32 * j + 8 * qd + 4 * fhalf;
-                    if (n < N) {
-                        u32x2 pk = {pack_bf16(acc[mi][j][4 * qd], acc[mi][j][4 * qd + 1]),
-                                    pack_bf16(acc[mi][j][4 * qd + 2], acc[mi][j][4 * qd + 3])};
-                        *reinterpret_cast<u32x2*>(crow + n) = pk;
-                    }
-                }
-            }
+        for (int ps = 0; ps < 32 * MT / RPP; ++ps) {
+            const int r = rr + RPP * ps;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(ep + r * RBW + ((cc ^ ((r >> KSH) & (CPR - 1))) << 4));
+            if (r < rows_here)
+                *reinterpret_cast<u32x4*>(g.c + (size_t)(row0 + wm * 32 * MT + r) * N + ncol0 + cc * 8) = v;
         }
     }
 }
