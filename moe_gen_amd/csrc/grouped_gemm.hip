@@ -237,10 +237,13 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
         else        { srow0 = (n0 >> 7) * KB; srow1 = min((n0 >> 7) + 1, (N >> 7) - 1) * KB; }
     }
 
-    u32x4 ra[1][NA], rb[1][NB];
-    float rs[1][2] = {{1.0f, 1.0f}};
-    constexpr int set = 0;
-    auto gload = [&](int kt) {
+    // PF register sets: global loads run PF tiles ahead of the LDS stores.  One set when the
+    // workgroup is compute bound (large M tiles); two for the small-M tiles that only stream
+    // weights (decode), where bytes in flight per CU are what limits the HBM rate.
+    constexpr int PF = (MT == 1) ? 2 : 1;
+    u32x4 ra[PF][NA], rb[PF][NB];
+    float rs[PF][2];
+    auto gload = [&](int kt, int set) {
         const size_t kofs = (size_t)kt * BK;
 #pragma unroll
         for (int i = 0; i < NA; ++i) ra[set][i] = gload16(g.a + (size_t)a_src[i] * K + kofs + lchunk * 8);
@@ -254,7 +257,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
             rs[set][1] = sc1[srow1 + (kt >> 1)];
         }
     };
-    auto lds_store = [&](uint8_t* As) {
+    auto lds_store = [&](uint8_t* As, int set) {
         uint8_t* Bs = As + A_STAGE;
 #pragma unroll
         for (int i = 0; i < NA; ++i) *reinterpret_cast<u32x4*>(As + a_lds + i * RA * ROW_B) = ra[set][i];
@@ -329,16 +332,20 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     };
 
     // ---- main loop ----
-    // On entry to iteration kt: LDS stage kt&1 holds tile kt and the registers hold tile kt+1
-    // (possibly still in flight).  The iteration moves tile kt+1 into the other LDS stage, refills
-    // the registers with tile kt+2 and multiplies tile kt.
+    // On entry to iteration kt: LDS stage kt&1 holds tile kt and the registers hold tiles kt+1 ..
+    // kt+PF (possibly still in flight).  The iteration moves tile kt+1 into the other LDS stage,
+    // refills that register set with tile kt+1+PF and multiplies tile kt.
     const int nk = K / BK;
-    gload(0);
-    lds_store(smem0);
-    if (nk > 1) gload(1);
+    gload(0, 0);
+    lds_store(smem0, 0);
+#pragma unroll
+    for (int d = 0; d < PF; ++d)
+        if (1 + d < nk) gload(1 + d, d);
     __syncthreads();
     const bool mfma_first = wave < 4;   // waves w and w+4 share a SIMD
-    for (int kt = 0; kt < nk; ++kt) {
+    // iteration kt: tile kt+1 is in register set kt % PF; it moves to the other LDS stage and the
+    // set is refilled with tile kt+1+PF (the loop is unrolled by PF so the set index is static)
+    auto iteration = [&](int kt, int set) {
         const uint8_t* rd = (kt & 1) ? smem1 : smem0;
         uint8_t* wr = (kt & 1) ? smem0 : smem1;
         // the wave that is multiplying outranks its SIMD partner that is moving data
@@ -346,17 +353,23 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
             __builtin_amdgcn_s_setprio(2);
             compute(rd, kt > 0);
             __builtin_amdgcn_s_setprio(0);
-            if (kt + 1 < nk) lds_store(wr);
-            if (kt + 2 < nk) gload(kt + 2);
+            if (kt + 1 < nk) lds_store(wr, set);
+            if (kt + 1 + PF < nk) gload(kt + 1 + PF, set);
         } else {
-            if (kt + 1 < nk) lds_store(wr);
-            if (kt + 2 < nk) gload(kt + 2);
+            if (kt + 1 < nk) lds_store(wr, set);
+            if (kt + 1 + PF < nk) gload(kt + 1 + PF, set);
             __builtin_amdgcn_s_setprio(2);
             compute(rd, kt > 0);
             __builtin_amdgcn_s_setprio(0);
         }
         __syncthreads();   // (waits for this wave's LDS reads and writes, then for the other waves)
+    };
+    int kt = 0;
+    for (; kt + PF <= nk; kt += PF) {
+#pragma unroll
+        for (int d = 0; d < PF; ++d) iteration(kt + d, d);
     }
+    if (PF == 2 && kt < nk) iteration(kt, 0);
     mfmas(LAST);
 
     // ---- epilogue ----
