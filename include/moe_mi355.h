@@ -207,6 +207,9 @@ int moe_combine(const void* y, const int32_t* pos, const int32_t* topk_idx, cons
  */
 typedef struct moe_stager moe_stager;
 
+enum { MOE_STAGE_CYCLIC = 0,       /* copy every module of the type in registration order (the reference's policy) */
+       MOE_STAGE_ON_DEMAND = 1     /* copy only what moe_stage_fetch / moe_stage_acquire name */ };
+
 enum { MOE_STAGE_DEVICE = 0,       /* slots are device memory, copies use hipMemcpyAsync */
        MOE_STAGE_HOST_MEMCPY = 1   /* slots are host memory, copies use memcpy: host-only tests */ };
 
@@ -228,6 +231,16 @@ int moe_stage_pump(moe_stager* s);
 int moe_stage_acquire(moe_stager* s, int32_t id, void* stream, int32_t* slot);
 /* free_weights_buffer: the slot may be overwritten once `stream` reaches this point. */
 int moe_stage_release(moe_stager* s, int32_t id, void* stream);
+/* Copy policy of a module type.  MOE_STAGE_ON_DEMAND turns the cyclic prefetch of that type
+ * off: the reference copies every expert of every layer whether or not a token was routed to
+ * it (HtoD_Engine.cpp:201-268 walks the whole queue); with the per-expert token counts of
+ * moe_dispatch on the host, a caller can stage only the experts that will run. */
+int moe_stage_set_policy(moe_stager* s, int32_t type, int32_t policy);
+/* Enqueue the copies of modules ids[0..n) that are not resident, in the given order (callers
+ * list the busiest experts first so the grouped kernel's first tiles have their weights
+ * earliest).  Fails with MOE_ERR_STATE when a module finds no free slot of its type;
+ * *n_enqueued (optional) receives the number of copies issued. */
+int moe_stage_fetch(moe_stager* s, const int32_t* ids, int32_t n, int32_t* n_enqueued);
 /* Whether module `id` currently occupies a slot (copied or copy in flight). */
 int moe_stage_resident(moe_stager* s, int32_t id);
 /* Grow (or shrink back) the number of usable slots of a type within the memory

@@ -46,6 +46,8 @@ SIGNATURES = {
                                    c_int32, c_int32, c_void_p, c_void_p]),
     "moe_stage_create": (ctypes.c_int, [ctypes.POINTER(c_void_p), c_int32, ctypes.POINTER(c_size_t),
                                         ctypes.POINTER(c_int32), ctypes.POINTER(c_void_p), c_int32]),
+    "moe_stage_set_policy": (ctypes.c_int, [c_void_p, c_int32, c_int32]),
+    "moe_stage_fetch": (ctypes.c_int, [c_void_p, ctypes.POINTER(c_int32), c_int32, ctypes.POINTER(c_int32)]),
     "moe_stage_add_module": (ctypes.c_int, [c_void_p, c_int32, c_int32, ctypes.POINTER(c_void_p),
                                             ctypes.POINTER(c_size_t), ctypes.POINTER(c_size_t)]),
     "moe_stage_pump": (ctypes.c_int, [c_void_p]),

@@ -140,9 +140,15 @@ def _tensors_of(expert, fetched=None):
     return (*ws, *ss)
 
 
-def collect_pointers(experts, cache):
+def collect_pointers(experts, cache, counts=None):
     """Pointer tables for a list of expert modules, plus the list of engine keys to release
     once the kernels that read the weights are enqueued.
+
+    counts: optional per-expert token counts (device int32 [E]).  When given and the engine can
+    stage on demand (it has `fetch`), only the experts with a non-zero count are copied, busiest
+    first, and the others get a placeholder pointer that no tile ever reads -- the reference
+    copies every expert of the layer blindly (HtoD_Engine.cpp:201-268).  Costs one host read of
+    E integers per call.
 
     Experts backed by an engine (an Expert_Wrapper-like object with `core_engine`,
     `get_weights=True` and `expert_weights_idx`) are fetched through
@@ -158,10 +164,24 @@ def collect_pointers(experts, cache):
         # behind by a skipped expert; one call reclaims what the previous layer left
         if getattr(first, "expert_idx", -1) != -1:
             first.core_engine.clear_expert_buffer(first.layer_idx, 0)
-        for ex in experts:
+        hot = None
+        if counts is not None and hasattr(first.core_engine, "fetch"):
+            c_host = counts.tolist()
+            hot = sorted((e for e in range(len(experts)) if c_host[e] > 0), key=lambda e: -c_host[e])
+            first.core_engine.fetch([experts[e].expert_weights_idx for e in hot])
+        if hot is None:
+            chosen = range(len(experts))
+        else:
+            chosen = hot or [0]                  # no routed token at all: one expert stands in
+        got = {}
+        for e in chosen:
+            ex = experts[e]
             fetched = ex.core_engine.get_weights(ex.expert_weights_idx)
             keys.append((ex.core_engine, ex.expert_weights_idx))
-            for c, t in zip(cols, _tensors_of(ex, fetched)):
+            got[e] = _tensors_of(ex, fetched)
+        stand_in = got[next(iter(chosen))]
+        for e in range(len(experts)):
+            for c, t in zip(cols, got.get(e, stand_in)):
                 c.append(t)
         fp8 = cols[0][0].dtype == FP8
         p = ops.expert_pointers(cols[0], cols[1], cols[2], *(cols[3:] if fp8 else (None, None, None)))
@@ -223,7 +243,8 @@ def moe_forward(block, hidden_states: torch.Tensor, spec: ops.RouterSpec, gate_w
         counts, offsets, perm, pos, xs = ops.dispatch(idx, E, None if fused_gather else x)
         row_map = torch.div(perm, k, rounding_mode="floor").to(torch.int32) if fused_gather else None
     block.last_counts = counts
-    ptrs, keys = collect_pointers(list(experts), cache.setdefault("routed", {}))
+    aware = counts if getattr(block, "routing_aware_staging", False) else None
+    ptrs, keys = collect_pointers(list(experts), cache.setdefault("routed", {}), aware)
     y = _grouped(timer, "routed", x if fused_gather else xs, row_map, ptrs, offsets, n * k)
     for eng, key in keys:
         eng.free_weights_buffer(key)

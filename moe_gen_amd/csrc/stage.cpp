@@ -14,8 +14,10 @@
 // no host thread exists and the host never waits: a copy is enqueued as soon as a slot
 // is free (pump), the consumer's stream waits on the copy's event (acquire), and the
 // next copy into a slot waits on the event recorded by the consumer when it let go of
-// the slot (release).  The copy order is the reference's: per type, the modules in the
-// order they were registered, cyclically, whether or not the router will use them.
+// the slot (release).  The default copy order is the reference's: per type, the modules in
+// the order they were registered, cyclically, whether or not the router will use them.
+// A type can instead be switched to on-demand: nothing is copied until the caller names the
+// modules it needs (fetch), typically the experts with a non-zero token count, busiest first.
 #include <cstring>
 #include <deque>
 #include <mutex>
@@ -46,6 +48,7 @@ struct Type {
     std::vector<char> freed_valid;
     std::vector<int> order;             // registration order
     std::deque<int> fifo;               // cyclic copy queue
+    int policy = MOE_STAGE_CYCLIC;
 };
 
 }  // namespace
@@ -67,16 +70,10 @@ int find_free(const Type& t) {
     return -1;
 }
 
-// one turn of the copy worker for one type; returns 1 if a copy was enqueued, 0 if not, <0 on error
-int pump_type(moe_stager* st, int ti) {
-    Type& t = st->types[ti];
-    if (t.fifo.empty()) return 0;
-    const int slot = find_free(t);
-    if (slot < 0) return 0;
-    const int id = t.fifo.front();
+// enqueue the copy of module `id` into free slot `slot` of its type
+int copy_into(moe_stager* st, int id, int slot) {
     Module& m = st->modules[id];
-    if (m.slot >= 0) return 0;  // next in line still occupies a slot: nothing to do until it is released
-    t.fifo.pop_front();
+    Type& t = st->types[m.type];
     uint8_t* dst = t.mem + (size_t)slot * t.slot_bytes;
     if (st->backend == MOE_STAGE_DEVICE) {
         if (t.freed_valid[slot]) {
@@ -93,8 +90,37 @@ int pump_type(moe_stager* st, int ti) {
     st->n_copies += 1;
     t.owner[slot] = id;
     m.slot = slot;
+    return MOE_OK;
+}
+
+// one turn of the copy worker for one type; returns 1 if a copy was enqueued, 0 if not, <0 on error
+int pump_type(moe_stager* st, int ti) {
+    Type& t = st->types[ti];
+    if (t.policy != MOE_STAGE_CYCLIC || t.fifo.empty()) return 0;
+    const int slot = find_free(t);
+    if (slot < 0) return 0;
+    const int id = t.fifo.front();
+    if (st->modules[id].slot >= 0) return 0;  // next in line still occupies a slot: nothing to do until it is released
+    t.fifo.pop_front();
+    int rc = copy_into(st, id, slot);
+    if (rc != MOE_OK) return rc;
     t.fifo.push_back(id);  // the reference pushes the name back for the next pass
     return 1;
+}
+
+// on-demand copy of one module; 1 if enqueued, 0 if already resident, <0 on error
+int fetch_one(moe_stager* st, int id) {
+    Module& m = st->modules[id];
+    if (m.slot >= 0) return 0;
+    Type& t = st->types[m.type];
+    const int slot = find_free(t);
+    if (slot < 0) {
+        moe::set_error("moe_stage_fetch: no free slot of type %d for module %d (%d active slots, all held)", m.type, id,
+                       t.n_active);
+        return MOE_ERR_STATE;
+    }
+    int rc = copy_into(st, id, slot);
+    return rc != MOE_OK ? rc : 1;
 }
 
 int pump_all(moe_stager* st) {
@@ -190,6 +216,10 @@ extern "C" int moe_stage_acquire(moe_stager* st, int32_t id, void* stream, int32
     std::lock_guard<std::mutex> lk(st->mu);
     MOE_REQUIRE(id >= 0 && id < (int)st->modules.size(), "moe_stage_acquire: unknown module id %d", id);
     Module& m = st->modules[id];
+    if (m.slot < 0 && st->types[m.type].policy == MOE_STAGE_ON_DEMAND) {
+        int r = fetch_one(st, id);
+        if (r < 0) return r;
+    }
     while (m.slot < 0) {
         int r = pump_all(st);
         if (r < 0) return r;
@@ -222,6 +252,34 @@ extern "C" int moe_stage_release(moe_stager* st, int32_t id, void* stream) {
     m.slot = -1;
     int r = pump_all(st);  // the worker refills a freed slot at once
     return r < 0 ? r : MOE_OK;
+}
+
+extern "C" int moe_stage_set_policy(moe_stager* st, int32_t type, int32_t policy) {
+    MOE_REQUIRE(st, "moe_stage_set_policy: NULL stager");
+    std::lock_guard<std::mutex> lk(st->mu);
+    MOE_REQUIRE(type >= 0 && type < (int)st->types.size(), "moe_stage_set_policy: bad type %d", type);
+    MOE_REQUIRE(policy == MOE_STAGE_CYCLIC || policy == MOE_STAGE_ON_DEMAND, "moe_stage_set_policy: bad policy %d",
+                policy);
+    st->types[type].policy = policy;
+    return MOE_OK;
+}
+
+extern "C" int moe_stage_fetch(moe_stager* st, const int32_t* ids, int32_t n, int32_t* n_enqueued) {
+    MOE_REQUIRE(st && (ids || n == 0), "moe_stage_fetch: NULL argument");
+    MOE_REQUIRE(n >= 0, "moe_stage_fetch: n %d < 0", n);
+    std::lock_guard<std::mutex> lk(st->mu);
+    int done = 0;
+    for (int i = 0; i < n; ++i) {
+        MOE_REQUIRE(ids[i] >= 0 && ids[i] < (int)st->modules.size(), "moe_stage_fetch: unknown module id %d", ids[i]);
+        int r = fetch_one(st, ids[i]);
+        if (r < 0) {
+            if (n_enqueued) *n_enqueued = done;
+            return r;
+        }
+        done += r;
+    }
+    if (n_enqueued) *n_enqueued = done;
+    return MOE_OK;
 }
 
 extern "C" int moe_stage_resident(moe_stager* st, int32_t id) {

@@ -113,6 +113,25 @@ class Stager:
         self.type_of[module_key] = module_type
         return mid
 
+    def set_policy(self, module_type: str, policy: str) -> None:
+        """"cyclic": every module of the type is copied in registration order whether or not it
+        will be used (the reference's worker, HtoD_Engine.cpp:201-268); "on_demand": only the
+        modules named by fetch() / get_weights() are copied."""
+        if policy not in ("cyclic", "on_demand"):
+            raise RuntimeError(f"unknown staging policy {policy!r}")
+        N.check(N.lib().moe_stage_set_policy(self._h, self.types.index(module_type), 1 if policy == "on_demand" else 0),
+                "moe_stage_set_policy")
+
+    def fetch(self, module_keys) -> int:
+        """Enqueue the copies of the listed modules that are not resident, in the given order;
+        returns how many copies were issued."""
+        ids = [self._id(k) for k in module_keys]
+        n = len(ids)
+        done = ctypes.c_int32(0)
+        N.check(N.lib().moe_stage_fetch(self._h, (ctypes.c_int32 * max(n, 1))(*ids), n, ctypes.byref(done)),
+                "moe_stage_fetch")
+        return done.value
+
     def pump(self) -> int:
         r = N.lib().moe_stage_pump(self._h)
         if r < 0:

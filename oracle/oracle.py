@@ -367,10 +367,32 @@ class SlotPoolModel:
         self.L = num_hidden_layers
         self.E = num_local_experts
         self.copies = []
+        self.on_demand = set()      # module types taken out of the cyclic queue
+
+    def fetch(self, names):
+        """On-demand staging (not in the reference, whose worker copies every module): copy
+        the listed modules that are not resident into the first empty slot of their type, in
+        the given order."""
+        type_of = {n: t for t, q in self.queues.items() for n in q}
+        done = 0
+        for name in names:
+            if name in self.resident:
+                continue
+            t = type_of[name]
+            if None not in self.slots[t]:
+                raise RuntimeError(f"no free slot of type {t} for {name}")
+            s = self.slots[t].index(None)
+            self.slots[t][s] = name
+            self.resident[name] = (t, s)
+            self.copies.append((name, t, s))
+            done += 1
+        return done
 
     def pump(self):
         did = False
         for t in self.queues:
+            if t in self.on_demand:
+                continue
             if None in self.slots[t] and self.queues[t]:
                 s = self.slots[t].index(None)
                 name = self.queues[t].pop(0)

@@ -145,3 +145,46 @@ def test_block_with_library_stager():
     assert torch.equal(out, ref)
     assert st.stats()[0] >= 3 * (w.E + 1)
     st.close()
+
+
+def test_block_with_routing_aware_staging():
+    """With per-expert token counts on the host, only experts that received tokens are staged
+    (busiest first); the output is bit-identical to resident weights and the copy count equals the
+    number of such experts.  The reference's worker copies every expert of the layer."""
+    from moe_gen_amd import StagedExpert, Stager, synthetic
+    w = synthetic.WORKLOADS["deepseek_v3_w8a16"].scaled(n=24, h=512, I=256, E=64, n_group=8, topk_group=4, k=4, seq=8)
+    blk = synthetic.build_block(w, device="cuda", gen_device="cpu")
+    x = synthetic.hidden_states(w, "cpu").cuda()
+    ref = blk(x).clone()
+    used = int((blk.last_counts > 0).sum())
+    assert 0 < used < w.E                                  # 24 tokens x 4 slots cannot reach all 64 experts
+    names = blk.experts[0].names
+    fp8 = torch.float8_e4m3fn
+    shapes = {"routed_expert": {f"{n}.weight": (tuple(getattr(blk.experts[0], n).weight.shape), fp8) for n in names},
+              "shared_expert": {f"{n}.weight": (tuple(getattr(blk.shared_experts, n).weight.shape), fp8) for n in names}}
+    st = Stager(shapes, {"routed_expert": w.E, "shared_expert": 1}, model_type="deepseek_v3", num_hidden_layers=8,
+                num_local_experts=w.E)
+    st.set_policy("routed_expert", "on_demand")
+    L = 5
+    wrapped = []
+    for e, ex in enumerate(blk.experts):
+        st.add_module(f"routed_expert_{L}_{e}", "routed_expert",
+                      {f"{n}.weight": getattr(ex, n).weight.data.cpu().pin_memory() for n in names})
+        scales = {f"{n}.weight_scale_inv": getattr(ex, n).weight_scale_inv.data for n in names}
+        for n in names:                                    # the resident copy is gone: a stale pointer would show
+            getattr(ex, n).weight.data = torch.zeros(1, dtype=fp8, device="cuda")
+        wrapped.append(StagedExpert(ex, L, e, st, scales))
+    sh = blk.shared_experts
+    st.add_module(f"shared_expert_{L}", "shared_expert", {f"{n}.weight": getattr(sh, n).weight.data.cpu().pin_memory() for n in names})
+    blk.experts = torch.nn.ModuleList(wrapped)
+    blk.shared_experts = StagedExpert(sh, L, -1, st, {f"{n}.weight_scale_inv": getattr(sh, n).weight_scale_inv.data for n in names})
+    blk.routing_aware_staging = True
+    assert st.pump() == 1                                  # the shared expert (cyclic) is prefetched; no routed expert
+    for rep in range(3):
+        c0 = st.stats()[0]
+        out = blk(x)
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref), rep
+        assert st.stats()[0] - c0 == used + 1, (rep, st.stats()[0] - c0, used)   # + the shared expert
+        assert not any(st.resident(f"routed_expert_{L}_{e}") for e in range(w.E))
+    st.close()

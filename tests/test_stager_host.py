@@ -101,3 +101,50 @@ def test_errors_and_phase_switch():
     assert big.pump() == 2 and big.resident("routed_expert_0_1") and not big.resident("routed_expert_0_2")
     with pytest.raises(RuntimeError):
         big.add_module("routed_expert_0_9", "routed_expert", {"gate_proj.weight": torch.zeros(1)})
+
+
+def test_on_demand_fetches_only_what_is_named():
+    """Routing-aware staging: with the on-demand policy nothing is copied until named; fetch()
+    copies the named modules in the given order into the first free slots, skips resident ones,
+    and fails when the pool is full.  Checked against the Python slot-pool model and by content."""
+    layers, E, slots = 2, 8, 5
+    st, model, host, names = make("mixtral", layers, E, slots, 0)
+    st.set_policy("routed_expert", "on_demand"); model.on_demand.add("routed_expert")
+    assert st.pump() == 1                                  # only the (cyclic) shared expert moves
+    while model.pump():
+        pass
+    assert not any(st.resident(k) for k in names["routed_expert"])
+    rng = torch.Generator().manual_seed(3)
+    for step in range(12):
+        L = step % layers
+        counts = torch.randint(0, 4, (E,), generator=rng) * (torch.rand(E, generator=rng) < 0.6)
+        hot = sorted((e for e in range(E) if counts[e] > 0), key=lambda e: -int(counts[e]))[:slots]
+        keys = [f"routed_expert_{L}_{e}" for e in hot]
+        assert st.fetch(keys) == model.fetch(keys) == len(keys)
+        assert st.fetch(keys) == 0                         # already resident: nothing to do
+        for k2 in names["routed_expert"]:
+            assert st.resident(k2) == (k2 in model.resident), (step, k2)
+        for key in keys:
+            w = st.get_weights(key)
+            assert all(torch.equal(w[n], host[key][n]) for n in w), key
+        for key in keys:
+            st.free_weights_buffer(key); model.release(key)
+        assert not any(st.resident(k) for k in names["routed_expert"])   # a freed slot is not refilled
+    assert st.stats()[0] == len(model.copies)
+    # get_weights on a module nobody fetched stages it alone
+    w = st.get_weights("routed_expert_1_7")
+    assert all(torch.equal(w[n], host["routed_expert_1_7"][n]) for n in w)
+    # pool exhausted: 4 more fit, the 5th does not
+    assert st.fetch([f"routed_expert_0_{e}" for e in range(4)]) == 4
+    with pytest.raises(RuntimeError, match="no free slot"):
+        st.fetch(["routed_expert_0_4", "routed_expert_0_5"])
+    with pytest.raises(RuntimeError, match="Module key not found"):
+        st.fetch(["routed_expert_9_9"])
+    with pytest.raises(RuntimeError, match="unknown staging policy"):
+        st.set_policy("routed_expert", "sometimes")
+    # back to the reference's policy: the queue resumes where it stood
+    for e in range(4):
+        st.free_weights_buffer(f"routed_expert_0_{e}")
+    st.free_weights_buffer("routed_expert_1_7")
+    st.set_policy("routed_expert", "cyclic")
+    assert st.pump() == slots and st.resident("routed_expert_0_0")
