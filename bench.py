@@ -120,13 +120,17 @@ def staged_run(w, blk, x, steps: int, routing_aware: bool = False):
     st.pump()
     step(0); step(1)
     torch.cuda.synchronize()
-    b0 = st.stats()[1]
+    c0, b0 = st.stats()
     t0 = _t.perf_counter()
     for i in range(steps):
         step(i)
     torch.cuda.synchronize()
     dt = _t.perf_counter() - t0
-    nbytes = st.stats()[1] - b0
+    copies, nbytes = st.stats()
+    if routing_aware:
+        per_step = (nbytes - b0) / steps           # on-demand copies are issued inside the step they serve
+    else:                                          # the cyclic prefetch runs ahead of the timed window
+        per_step = nbytes / copies * (E + (1 if has_shared else 0))
     blk.routing_aware_staging = False
     blk.experts = resident_experts
     if has_shared:
@@ -136,7 +140,7 @@ def staged_run(w, blk, x, steps: int, routing_aware: bool = False):
             if routing_aware else
             "all expert weights re-staged from pinned host memory every step (the reference's policy)")
     return {"tokens_per_s": w.n * steps / dt, "ms_per_step": dt * 1e3 / steps,
-            "host_to_hbm_gib_per_step": nbytes / steps / 2 ** 30,
+            "host_to_hbm_gib_per_step": per_step / 2 ** 30,
             "note": note + "; bounded by the host link, not by the kernels"}
 
 
