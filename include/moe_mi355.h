@@ -185,6 +185,29 @@ int moe_combine(const void* y, const int32_t* pos, const int32_t* topk_idx, cons
                 const void* shared, int32_t n_tokens, int32_t top_k, int32_t hidden,
                 int32_t mode, void* out, void* stream);
 
+/* ------------------------------------------------- the step either side of the block */
+
+/*
+ * post_attention_layernorm, the op that produces the block's input
+ * (DeepseekV3RMSNorm.forward, modeling_deepseek_v3.py:125-150; V2 :127-134; call site :1363):
+ *     out = bf16( weight * bf16( f32(x) * rsqrt(mean(f32(x)^2) + eps) ) )
+ * in one kernel.  x, out device bf16 [n, h] (out != x); weight device bf16 [h]; h % 8 == 0.
+ */
+int moe_rmsnorm(const void* x, const void* weight, float eps, int32_t n_tokens, int32_t hidden,
+                void* out, void* stream);
+
+/*
+ * moe_combine followed by the decoder layer's residual add
+ * (hidden_states = residual + hidden_states, modeling_deepseek_v3.py:1365) in the same pass:
+ *     out[t] = bf16( f32(residual[t]) + f32(<moe_combine result>[t]) )
+ *   residual device bf16 [n, h]; may be the same buffer as out (in-place update of the
+ *   residual stream).  Other arguments as moe_combine.
+ */
+int moe_combine_residual(const void* y, const int32_t* pos, const int32_t* topk_idx,
+                         const float* topk_w, const void* shared, const void* residual,
+                         int32_t n_tokens, int32_t top_k, int32_t hidden, int32_t mode,
+                         void* out, void* stream);
+
 /* ------------------------------------------------- expert-weight staging */
 
 /*

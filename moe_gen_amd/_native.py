@@ -44,6 +44,9 @@ SIGNATURES = {
     "moe_dequant_fp8_block128": (ctypes.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p]),
     "moe_combine": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32,
                                    c_int32, c_int32, c_void_p, c_void_p]),
+    "moe_combine_residual": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32,
+                                            c_int32, c_int32, c_int32, c_void_p, c_void_p]),
+    "moe_rmsnorm": (ctypes.c_int, [c_void_p, c_void_p, ctypes.c_float, c_int32, c_int32, c_void_p, c_void_p]),
     "moe_stage_create": (ctypes.c_int, [ctypes.POINTER(c_void_p), c_int32, ctypes.POINTER(c_size_t),
                                         ctypes.POINTER(c_int32), ctypes.POINTER(c_void_p), c_int32]),
     "moe_stage_set_policy": (ctypes.c_int, [c_void_p, c_int32, c_int32]),

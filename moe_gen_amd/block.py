@@ -231,6 +231,11 @@ def moe_forward(block, hidden_states: torch.Tensor, spec: ops.RouterSpec, gate_w
         x = x.contiguous()
     n, h = x.shape
     k, E = spec.top_k, spec.n_experts
+    residual = None
+    fuse = getattr(block, "_norm_residual", None)
+    if fuse is not None:                      # see norm_moe_residual
+        residual = x
+        x = ops.rmsnorm(x, fuse[0], fuse[1])
     cache = block.__dict__.setdefault("_moe_cache", {})
     gw = _gate_weight_bf16(gate_weight, cache)
     b = None if bias is None else bias.data.to(torch.float32)
@@ -259,5 +264,26 @@ def moe_forward(block, hidden_states: torch.Tensor, spec: ops.RouterSpec, gate_w
         for eng, key in skeys:
             eng.free_weights_buffer(key)
     with _span(timer, "combine"):
-        out = ops.combine(y, pos, idx, w, sh, combine_mode)
+        out = ops.combine(y, pos, idx, w, sh, combine_mode, residual=residual)
     return out.view(*shape), logits
+
+
+@torch.no_grad()
+def norm_moe_residual(block, hidden_states: torch.Tensor, norm_weight: torch.Tensor, eps: float = 1e-6):
+    """The MLP half of the reference decoder layer around an MoE block
+    (modeling_deepseek_v3.py:1361-1365, modeling_deepseek_v2.py:1522-1526):
+
+        residual = hidden_states
+        hidden_states = post_attention_layernorm(hidden_states)
+        hidden_states = mlp(hidden_states)
+        hidden_states = residual + hidden_states
+
+    with the norm as one kernel and the residual add folded into the combine's output pass.
+    Returns what `block(...)` returns with the new residual stream in place of the block output
+    (Mixtral: a tuple with the router logits second)."""
+    w = norm_weight.data if isinstance(norm_weight, torch.nn.Parameter) else norm_weight
+    block._norm_residual = (w, float(eps))
+    try:
+        return block(hidden_states)
+    finally:
+        block._norm_residual = None

@@ -6,7 +6,8 @@
 //        (new_x.view(n,k,h).float() * w[...,None]).sum(1).to(bf16)
 //   V2  modeling_deepseek_v2.py:744-757:  same with w cast to bf16 first (bf16 products)
 //   Mixtral (transformers 4.42.0): final.index_add_(0, top_x, expert_out * w) per expert
-// and `y = y + self.shared_experts(identity)` (modeling_deepseek_v3.py:624-625).
+// and `y = y + self.shared_experts(identity)` (modeling_deepseek_v3.py:624-625); optionally also the
+// decoder layer's `hidden_states = residual + hidden_states` that follows the block (:1365).
 // The reference materialises new_x [n,k,h] (and an fp32 copy of it); here each
 // output element is accumulated in a register from the k source rows.
 //
@@ -23,7 +24,7 @@ template <int MODE>
 __global__ __launch_bounds__(256) void combine_kernel(const u32x4* __restrict__ y, const int32_t* __restrict__ pos,
                                                       const int32_t* __restrict__ topk_idx,
                                                       const float* __restrict__ topk_w, const u32x4* __restrict__ shared,
-                                                      int k, int chunks, u32x4* __restrict__ out) {
+                                                      const u32x4* residual, int k, int chunks, u32x4* out) {
     __shared__ int s_row[MAX_K];
     __shared__ float s_w[MAX_K];
     const int t = blockIdx.x;
@@ -75,6 +76,15 @@ __global__ __launch_bounds__(256) void combine_kernel(const u32x4* __restrict__ 
             }
             o[i] = lo | (hi << 16);
         }
+        if (residual) {  // may alias out: this thread reads its 16 bytes before it writes them
+            const u32x4 r = residual[(size_t)t * chunks + c];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t lo = f32_to_bf16_bits(__uint_as_float(r[i] << 16) + __uint_as_float(o[i] << 16));
+                const uint32_t hi = f32_to_bf16_bits(__uint_as_float(r[i] & 0xffff0000u) + __uint_as_float(o[i] & 0xffff0000u));
+                o[i] = lo | (hi << 16);
+            }
+        }
         out[(size_t)t * chunks + c] = o;
     }
 }
@@ -82,29 +92,49 @@ __global__ __launch_bounds__(256) void combine_kernel(const u32x4* __restrict__ 
 }  // namespace
 }  // namespace moe
 
-extern "C" int moe_combine(const void* y, const int32_t* pos, const int32_t* topk_idx, const float* topk_w,
-                           const void* shared, int32_t n_tokens, int32_t top_k, int32_t hidden, int32_t mode,
-                           void* out, void* stream) {
-    using namespace moe;
-    MOE_REQUIRE(n_tokens >= 0, "moe_combine: n_tokens %d < 0", n_tokens);
+namespace moe {
+namespace {
+int combine_impl(const void* y, const int32_t* pos, const int32_t* topk_idx, const float* topk_w, const void* shared,
+                 const void* residual, int32_t n_tokens, int32_t top_k, int32_t hidden, int32_t mode, void* out,
+                 void* stream, const char* who) {
+    MOE_REQUIRE(n_tokens >= 0, "%s: n_tokens %d < 0", who, n_tokens);
     if (n_tokens == 0) return MOE_OK;
-    MOE_REQUIRE(y && pos && topk_w && out, "moe_combine: NULL tensor pointer");
-    MOE_REQUIRE(top_k >= 1 && top_k <= MAX_K, "moe_combine: top_k %d outside [1,%d]", top_k, MAX_K);
-    MOE_REQUIRE(hidden > 0 && hidden % 8 == 0, "moe_combine: hidden %d must be a positive multiple of 8", hidden);
-    MOE_REQUIRE(mode >= MOE_COMBINE_F32 && mode <= MOE_COMBINE_BF16_SEQ, "moe_combine: bad mode %d", mode);
-    MOE_REQUIRE(mode != MOE_COMBINE_BF16_SEQ || topk_idx, "moe_combine: topk_idx is required for MOE_COMBINE_BF16_SEQ");
+    MOE_REQUIRE(y && pos && topk_w && out, "%s: NULL tensor pointer", who);
+    MOE_REQUIRE(top_k >= 1 && top_k <= MAX_K, "%s: top_k %d outside [1,%d]", who, top_k, MAX_K);
+    MOE_REQUIRE(hidden > 0 && hidden % 8 == 0, "%s: hidden %d must be a positive multiple of 8", who, hidden);
+    MOE_REQUIRE(mode >= MOE_COMBINE_F32 && mode <= MOE_COMBINE_BF16_SEQ, "%s: bad mode %d", who, mode);
+    MOE_REQUIRE(mode != MOE_COMBINE_BF16_SEQ || topk_idx, "%s: topk_idx is required for MOE_COMBINE_BF16_SEQ", who);
+    MOE_REQUIRE(out != y && out != shared, "%s: out must not alias y or shared", who);
     hipStream_t st = as_stream(stream);
     dim3 grid(n_tokens), block(256);
     const u32x4* yv = static_cast<const u32x4*>(y);
     const u32x4* sv = static_cast<const u32x4*>(shared);
+    const u32x4* rv = static_cast<const u32x4*>(residual);
     u32x4* ov = static_cast<u32x4*>(out);
     const int chunks = hidden / 8;
     if (mode == MOE_COMBINE_F32)
-        hipLaunchKernelGGL(combine_kernel<MOE_COMBINE_F32>, grid, block, 0, st, yv, pos, topk_idx, topk_w, sv, top_k, chunks, ov);
+        hipLaunchKernelGGL(combine_kernel<MOE_COMBINE_F32>, grid, block, 0, st, yv, pos, topk_idx, topk_w, sv, rv, top_k, chunks, ov);
     else if (mode == MOE_COMBINE_BF16_PROD)
-        hipLaunchKernelGGL(combine_kernel<MOE_COMBINE_BF16_PROD>, grid, block, 0, st, yv, pos, topk_idx, topk_w, sv, top_k, chunks, ov);
+        hipLaunchKernelGGL(combine_kernel<MOE_COMBINE_BF16_PROD>, grid, block, 0, st, yv, pos, topk_idx, topk_w, sv, rv, top_k, chunks, ov);
     else
-        hipLaunchKernelGGL(combine_kernel<MOE_COMBINE_BF16_SEQ>, grid, block, 0, st, yv, pos, topk_idx, topk_w, sv, top_k, chunks, ov);
+        hipLaunchKernelGGL(combine_kernel<MOE_COMBINE_BF16_SEQ>, grid, block, 0, st, yv, pos, topk_idx, topk_w, sv, rv, top_k, chunks, ov);
     MOE_HIP_CHECK(hipGetLastError());
     return MOE_OK;
+}
+}  // namespace
+}  // namespace moe
+
+extern "C" int moe_combine(const void* y, const int32_t* pos, const int32_t* topk_idx, const float* topk_w,
+                           const void* shared, int32_t n_tokens, int32_t top_k, int32_t hidden, int32_t mode,
+                           void* out, void* stream) {
+    return moe::combine_impl(y, pos, topk_idx, topk_w, shared, nullptr, n_tokens, top_k, hidden, mode, out, stream,
+                             "moe_combine");
+}
+
+extern "C" int moe_combine_residual(const void* y, const int32_t* pos, const int32_t* topk_idx, const float* topk_w,
+                                    const void* shared, const void* residual, int32_t n_tokens, int32_t top_k,
+                                    int32_t hidden, int32_t mode, void* out, void* stream) {
+    MOE_REQUIRE(residual || n_tokens == 0, "moe_combine_residual: NULL residual");
+    return moe::combine_impl(y, pos, topk_idx, topk_w, shared, residual, n_tokens, top_k, hidden, mode, out, stream,
+                             "moe_combine_residual");
 }

@@ -1,0 +1,71 @@
+// RMSNorm ahead of the MoE block for gfx950: the reference's post_attention_layernorm,
+//   DeepseekV3RMSNorm.forward  modeling_deepseek_v3.py:125-150
+//   DeepseekV2RMSNorm.forward  modeling_deepseek_v2.py:127-134
+//     xf = x.float(); var = xf.pow(2).mean(-1); y = (xf * rsqrt(var + eps)).to(bf16); out = weight * y
+// in one pass over the row (the reference runs five elementwise/reduction kernels and three
+// host-synchronising isnan/isinf checks).  HBM bound: 2nh bytes in, 2nh bytes out.
+//
+// One wave per row, 16 bytes (8 bf16) per lane per step.  Summation order (shared with the CPU
+// checker): lane l adds the squares of chunks l, l+64, ... in ascending order, then a xor
+// butterfly 32..1; var = sum / h; rstd = 1 / sqrt(var + eps), sqrt and divide correctly rounded.
+// The row is read a second time for the scaling pass; it is at most a few tens of KB and still in
+// cache.
+#include "common.h"
+
+namespace moe {
+namespace {
+
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const u32x4* __restrict__ x, const u32x4* __restrict__ w,
+                                                      float eps, int n, int chunks, u32x4* __restrict__ out) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int row = blockIdx.x * 4 + wave;
+    if (row >= n) return;
+    const u32x4* xr = x + (size_t)row * chunks;
+    float acc = 0.0f;
+    for (int c = lane; c < chunks; c += 64) {
+        const u32x4 v = xr[c];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float lo = __uint_as_float(v[i] << 16), hi = __uint_as_float(v[i] & 0xffff0000u);
+            acc = acc + lo * lo;
+            acc = acc + hi * hi;
+        }
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) acc = acc + __shfl_xor(acc, m);
+    const float var = acc / (float)(chunks * 8);
+    const float rstd = 1.0f / __fsqrt_rn(var + eps);
+    u32x4* orow = out + (size_t)row * chunks;
+    for (int c = lane; c < chunks; c += 64) {
+        const u32x4 v = xr[c], g = w[c];
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float lo = round_to_bf16(__uint_as_float(v[i] << 16) * rstd);
+            const float hi = round_to_bf16(__uint_as_float(v[i] & 0xffff0000u) * rstd);
+            const uint32_t a = f32_to_bf16_bits(__uint_as_float(g[i] << 16) * lo);
+            const uint32_t b = f32_to_bf16_bits(__uint_as_float(g[i] & 0xffff0000u) * hi);
+            o[i] = a | (b << 16);
+        }
+        orow[c] = o;
+    }
+}
+
+}  // namespace
+}  // namespace moe
+
+extern "C" int moe_rmsnorm(const void* x, const void* weight, float eps, int32_t n_tokens, int32_t hidden, void* out,
+                           void* stream) {
+    using namespace moe;
+    MOE_REQUIRE(n_tokens >= 0, "moe_rmsnorm: n_tokens %d < 0", n_tokens);
+    if (n_tokens == 0) return MOE_OK;
+    MOE_REQUIRE(x && weight && out, "moe_rmsnorm: NULL tensor pointer");
+    MOE_REQUIRE(x != out, "moe_rmsnorm: out must not alias x (the row is read twice)");
+    MOE_REQUIRE(hidden > 0 && hidden % 8 == 0, "moe_rmsnorm: hidden %d must be a positive multiple of 8", hidden);
+    MOE_REQUIRE(eps >= 0.0f, "moe_rmsnorm: eps %g < 0", (double)eps);
+    hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)((n_tokens + 3) / 4)), dim3(256), 0, as_stream(stream),
+                       static_cast<const u32x4*>(x), static_cast<const u32x4*>(weight), eps, n_tokens, hidden / 8,
+                       static_cast<u32x4*>(out));
+    MOE_HIP_CHECK(hipGetLastError());
+    return MOE_OK;
+}

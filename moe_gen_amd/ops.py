@@ -196,8 +196,10 @@ def dequant_fp8_block128(q: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
 
 
 def combine(y: torch.Tensor, pos: torch.Tensor, topk_idx, topk_w: torch.Tensor, shared, mode: int,
-            out: torch.Tensor | None = None):
-    """out[t] = sum_j w[t,j] * y[pos[t*k+j]] (+ shared[t]); y bf16 [n*k,h] in sorted-row order."""
+            out: torch.Tensor | None = None, residual: torch.Tensor | None = None):
+    """out[t] = sum_j w[t,j] * y[pos[t*k+j]] (+ shared[t]); y bf16 [n*k,h] in sorted-row order.
+    residual: optional bf16 [n,h] added last (the decoder layer's `residual + hidden_states`,
+    modeling_deepseek_v3.py:1365); `out` may be the residual buffer itself."""
     n, k = topk_w.shape
     h = y.shape[1]
     _need(y, torch.bfloat16, "y", (n * k, h))
@@ -207,9 +209,29 @@ def combine(y: torch.Tensor, pos: torch.Tensor, topk_idx, topk_w: torch.Tensor, 
         _need(topk_idx, torch.int32, "topk_idx", (n, k))
     if shared is not None:
         _need(shared, torch.bfloat16, "shared", (n, h))
+    if residual is not None:
+        _need(residual, torch.bfloat16, "residual", (n, h))
     if out is None:
         out = torch.empty((n, h), dtype=torch.bfloat16, device=y.device)
     _need(out, torch.bfloat16, "out", (n, h))
-    N.check(N.lib().moe_combine(_ptr(y), _ptr(pos), _ptr(topk_idx), _ptr(topk_w), _ptr(shared), n, k, h, mode,
-                                _ptr(out), _stream()), "moe_combine")
+    L = N.lib()
+    if residual is None:
+        N.check(L.moe_combine(_ptr(y), _ptr(pos), _ptr(topk_idx), _ptr(topk_w), _ptr(shared), n, k, h, mode,
+                              _ptr(out), _stream()), "moe_combine")
+    else:
+        N.check(L.moe_combine_residual(_ptr(y), _ptr(pos), _ptr(topk_idx), _ptr(topk_w), _ptr(shared),
+                                       _ptr(residual), n, k, h, mode, _ptr(out), _stream()), "moe_combine_residual")
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, out: torch.Tensor | None = None):
+    """post_attention_layernorm (DeepseekV3RMSNorm.forward, modeling_deepseek_v3.py:125-150):
+    x bf16 [n,h], weight bf16 [h] -> bf16 [n,h]."""
+    _need(x, torch.bfloat16, "x")
+    n, h = x.shape
+    _need(weight, torch.bfloat16, "weight", (h,))
+    if out is None:
+        out = torch.empty_like(x)
+    _need(out, torch.bfloat16, "out", (n, h))
+    N.check(N.lib().moe_rmsnorm(_ptr(x), _ptr(weight), float(eps), n, h, _ptr(out), _stream()), "moe_rmsnorm")
     return out

@@ -422,6 +422,51 @@ int orc_combine(const uint16_t* ys, const int32_t* pos, const int32_t* idx, cons
 }
 
 /* ------------------------------------------------------------------ */
+/* the step either side of the block                                   */
+/* ------------------------------------------------------------------ */
+
+/* post_attention_layernorm: DeepseekV3RMSNorm.forward (modeling_deepseek_v3.py:125-150),
+ * DeepseekV2RMSNorm.forward (modeling_deepseek_v2.py:127-134):
+ *   xf = f32(x); var = mean(xf^2); y = bf16(xf * rsqrt(var + eps)); out = bf16(w * y)
+ * torch leaves the summation order of the mean and the accuracy of rsqrt to the
+ * backend; canonical choice here: squares summed in 64 strided partials over
+ * 8-element chunks (lane = chunk mod 64, ascending inside a lane), xor butterfly,
+ * var = sum / h, rstd = 1 / sqrt(var + eps) with correctly rounded sqrt and divide. */
+void orc_rmsnorm(const uint16_t* x, const uint16_t* w, float eps, int n, int h, uint16_t* out) {
+    const int chunks = h / 8;
+    for (int t = 0; t < n; ++t) {
+        const uint16_t* xr = x + (size_t)t * h;
+        float p[64];
+        for (int l = 0; l < 64; ++l) {
+            float a = 0.0f;
+            for (int c = l; c < chunks; c += 64)
+                for (int i = 0; i < 8; ++i) {
+                    float f = orc_bf16_to_f32(xr[c * 8 + i]);
+                    a = a + f * f;
+                }
+            p[l] = a;
+        }
+        for (int m = 32; m >= 1; m >>= 1) {
+            float q[64];
+            for (int l = 0; l < 64; ++l) q[l] = p[l] + p[l ^ m];
+            memcpy(p, q, sizeof p);
+        }
+        const float var = p[0] / (float)h;
+        const float rstd = 1.0f / sqrtf(var + eps);
+        for (int c = 0; c < h; ++c) {
+            float y = orc_bf16_to_f32(orc_f32_to_bf16(orc_bf16_to_f32(xr[c]) * rstd));
+            out[(size_t)t * h + c] = orc_f32_to_bf16(orc_bf16_to_f32(w[c]) * y);
+        }
+    }
+}
+
+/* hidden_states = residual + hidden_states (modeling_deepseek_v3.py:1365): bf16 + bf16 -> bf16 */
+void orc_add_residual(const uint16_t* a, const uint16_t* residual, int64_t n, uint16_t* out) {
+    for (int64_t i = 0; i < n; ++i)
+        out[i] = orc_f32_to_bf16(orc_bf16_to_f32(a[i]) + orc_bf16_to_f32(residual[i]));
+}
+
+/* ------------------------------------------------------------------ */
 /* bulk conversions for the numpy side                                 */
 /* ------------------------------------------------------------------ */
 

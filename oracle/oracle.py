@@ -271,6 +271,29 @@ def combine(ys_bf16, pos, idx, w, shared_bf16=None, mode=COMBINE_F32):
     return out
 
 
+def rmsnorm(x_bf16, w_bf16, eps: float = 1e-6) -> np.ndarray:
+    """post_attention_layernorm (modeling_deepseek_v3.py:125-150): bf16 [n,h] -> bf16 [n,h]."""
+    x = _c(x_bf16, np.uint16)
+    w = _c(w_bf16, np.uint16)
+    n, h = x.shape
+    if h % 8 or w.shape != (h,):
+        raise ValueError("rmsnorm: hidden size must be a multiple of 8 and match the weight")
+    out = np.empty((n, h), np.uint16)
+    lib().orc_rmsnorm(_p(x), _p(w), ctypes.c_float(eps), n, h, _p(out))
+    return out
+
+
+def add_residual(a_bf16, residual_bf16) -> np.ndarray:
+    """residual + hidden_states in bf16 (modeling_deepseek_v3.py:1365)."""
+    a = _c(a_bf16, np.uint16)
+    r = _c(residual_bf16, np.uint16)
+    if a.shape != r.shape:
+        raise ValueError("add_residual: shape mismatch")
+    out = np.empty(a.shape, np.uint16)
+    lib().orc_add_residual(_p(a), _p(r), ctypes.c_int64(a.size), _p(out))
+    return out
+
+
 # ----------------------------------------------------------------------------
 # expert MLP and the whole layer
 # ----------------------------------------------------------------------------

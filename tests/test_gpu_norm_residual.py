@@ -1,0 +1,91 @@
+"""GPU parity of the steps either side of the block: RMSNorm kernel, residual add folded into the
+combine, and the fused decoder-layer half against its unfused composition."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from test_gpu_dispatch_combine import rand_idx
+from util import bits
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("n,h,scale", [(1, 8, 1.0), (3, 64, 1.0), (130, 2048, 1.0), (257, 7168, 20.0), (64, 4096, 1e-3),
+                                       (5, 5120, 1.0), (9, 6144, 1.0)])
+def test_rmsnorm_bit_exact(n, h, scale):
+    from moe_gen_amd import ops
+    print(f"rmsnorm n={n} h={h} scale={scale}", flush=True)
+    g = torch.Generator().manual_seed(n + h)
+    x = (torch.randn(n, h, generator=g) * scale).to(torch.bfloat16)
+    x[0, : min(h, 16)] = 0
+    w = (1.0 + 0.2 * torch.randn(h, generator=g)).to(torch.bfloat16)
+    for eps in (1e-6, 1e-5):
+        out = ops.rmsnorm(x.cuda(), w.cuda(), eps)
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(out), O.rmsnorm(bits(x), bits(w), eps)), (n, h, eps)
+
+
+def test_rmsnorm_edges_and_errors():
+    from moe_gen_amd import ops
+    w = torch.ones(64, dtype=torch.bfloat16, device="cuda")
+    assert ops.rmsnorm(torch.zeros(0, 64, dtype=torch.bfloat16, device="cuda"), w).shape == (0, 64)
+    z = ops.rmsnorm(torch.zeros(6, 64, dtype=torch.bfloat16, device="cuda"), w)
+    assert not z.any()
+    x = torch.randn(4, 64, device="cuda").to(torch.bfloat16)
+    with pytest.raises(RuntimeError, match="alias"):
+        ops.rmsnorm(x, w, out=x)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        ops.rmsnorm(torch.zeros(2, 12, dtype=torch.bfloat16, device="cuda"), torch.ones(12, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(TypeError):
+        ops.rmsnorm(x.float(), w)
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2])
+@pytest.mark.parametrize("n,k,h,shared,inplace", [(1, 1, 8, False, False), (50, 2, 64, False, True),
+                                                  (257, 6, 2048, True, True), (100, 8, 7168, True, False)])
+def test_combine_residual_bit_exact(mode, n, k, h, shared, inplace):
+    from moe_gen_amd import ops
+    print(f"combine_residual mode={mode} n={n} k={k} h={h} shared={shared} inplace={inplace}", flush=True)
+    E = 16
+    idx = rand_idx(n, k, E, 7 * n + k)
+    _, _, perm, pos = O.dispatch(idx, E)
+    g = torch.Generator().manual_seed(n + mode)
+    ys = torch.randn(n * k, h, generator=g).to(torch.bfloat16)
+    w = torch.rand(n, k, generator=g) * 2.5
+    sh = torch.randn(n, h, generator=g).to(torch.bfloat16) if shared else None
+    res = (torch.randn(n, h, generator=g) * 8).to(torch.bfloat16)
+    res_d = res.cuda()
+    out = ops.combine(ys.cuda(), torch.from_numpy(pos).cuda(), torch.from_numpy(idx).cuda(), w.cuda(),
+                      None if sh is None else sh.cuda(), mode, out=res_d if inplace else None, residual=res_d)
+    torch.cuda.synchronize()
+    if inplace:
+        assert out.data_ptr() == res_d.data_ptr()
+    plain = O.combine(bits(ys), pos, idx, w.numpy(), None if sh is None else bits(sh), mode)
+    assert np.array_equal(bits(out), O.add_residual(plain, bits(res)))
+
+
+@pytest.mark.parametrize("name", ["deepseek_v3_w8a16", "deepseek_v2_lite", "mixtral_8x7b"])
+def test_fused_decoder_half_equals_composition(name):
+    """norm_moe_residual == residual + block(rmsnorm(residual)), bit for bit, and the norm it feeds
+    the block is the oracle's."""
+    from moe_gen_amd import norm_moe_residual, ops, synthetic
+    w = synthetic.WORKLOADS[name].scaled(n=192, h=512, I=256, seq=64)
+    blk = synthetic.build_block(w, device="cuda", gen_device="cpu")
+    stream_in = (synthetic.hidden_states(w, "cpu") * 3).cuda()
+    g = torch.Generator().manual_seed(5)
+    ln = (1.0 + 0.1 * torch.randn(w.h, generator=g)).to(torch.bfloat16).cuda()
+    xn = ops.rmsnorm(stream_in.view(-1, w.h), ln, 1e-6).view_as(stream_in)
+    assert np.array_equal(bits(xn.view(-1, w.h)), O.rmsnorm(bits(stream_in.view(-1, w.h)), bits(ln), 1e-6))
+    ref = blk(xn)
+    fused = norm_moe_residual(blk, stream_in, ln, 1e-6)
+    if isinstance(ref, tuple):
+        assert torch.equal(fused[1], ref[1])
+        ref, fused = ref[0], fused[0]
+    torch.cuda.synchronize()
+    assert fused.shape == stream_in.shape
+    assert np.array_equal(bits(fused.view(-1, w.h)), O.add_residual(bits(ref.view(-1, w.h)), bits(stream_in.view(-1, w.h))))
+    assert torch.equal(fused, stream_in + ref)
+    assert getattr(blk, "_norm_residual", None) is None      # a later plain call is the plain block
+    again = blk(xn)
+    assert torch.equal(again[0] if isinstance(again, tuple) else again, ref)
