@@ -144,6 +144,50 @@ def staged_run(w, blk, x, steps: int, routing_aware: bool = False):
             "note": note + "; bounded by the host link, not by the kernels"}
 
 
+def decoder_half_run(w, blk, x, steps: int):
+    """The MLP half of a decoder layer around the block (post-attention RMSNorm, block, residual
+    add): the library's fused form (one norm kernel, residual folded into the combine) against
+    the same block with the norm and the add as separate passes."""
+    import time as _t
+
+    import torch
+    from moe_gen_amd import norm_moe_residual, ops
+    from moe_gen_amd.block import StageTimer
+
+    ln = torch.ones(w.h, dtype=torch.bfloat16, device=x.device)
+    first = lambda r: r[0] if isinstance(r, tuple) else r
+
+    def fused():
+        return first(norm_moe_residual(blk, x, ln, 1e-6))
+
+    def separate():
+        xn = ops.rmsnorm(x.view(-1, w.h), ln, 1e-6).view_as(x)
+        return x + first(blk(xn))
+
+    out = {}
+    for name, fn in (("fused", fused), ("separate", separate)):
+        fn(); fn()
+        torch.cuda.synchronize()
+        t0 = _t.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        out[name + "_ms_per_step"] = (_t.perf_counter() - t0) * 1e3 / steps
+    timer = StageTimer()
+    blk.stage_timer = timer
+    for _ in range(steps):
+        fused()
+    torch.cuda.synchronize()
+    blk.stage_timer = None
+    st = {k: sum(v) / len(v) for k, v in timer.totals_ms().items()}
+    nh2 = 2.0 * w.n * w.h
+    out["rmsnorm_ms"] = st["rmsnorm"]
+    out["rmsnorm_gbps"] = 2 * nh2 / (st["rmsnorm"] * 1e-3) / 1e9            # read x, write the normalised copy
+    out["combine_residual_ms"] = st["combine"]
+    out["combine_residual_gbps"] = (w.combine_bytes + nh2) / (st["combine"] * 1e-3) / 1e9
+    return out
+
+
 # HBM traffic per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (two runs; FETCH_SIZE scaled by 2.0, the factor a plain copy kernel of known size showed on this
 # box, WRITE_SIZE by 1.0).  bench.py cannot run the profiler on itself, so the figures are recorded
@@ -225,6 +269,8 @@ def run_workload(name: str, args, with_cpu: bool):
                                          "combine": w.combine_bytes / (st["combine"] * 1e-3) / 1e9 / PEAK_HBM_GBPS}},
         "stage_ms": st,
     }
+    if args.decoder_half:
+        result["decoder_half"] = decoder_half_run(w, blk, x, args.steps)
     if args.staged:
         result["staged"] = staged_run(w, blk, x, max(2, args.steps // 2))
         result["staged_routing_aware"] = staged_run(w, blk, x, max(2, args.steps // 2), routing_aware=True)
@@ -247,6 +293,7 @@ def main():
                     "reading them through the row map inside the GEMM")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--staged", action="store_true", help="also time the block with weights staged from pinned host memory")
+    ap.add_argument("--decoder-half", action="store_true", help="also time RMSNorm + block + residual add, fused and separate")
     ap.add_argument("--cpu-sample", type=int, default=128)
     args = ap.parse_args()
     if args.gpus != 1:

@@ -233,13 +233,14 @@ def moe_forward(block, hidden_states: torch.Tensor, spec: ops.RouterSpec, gate_w
     k, E = spec.top_k, spec.n_experts
     residual = None
     fuse = getattr(block, "_norm_residual", None)
+    timer = getattr(block, "stage_timer", None)
     if fuse is not None:                      # see norm_moe_residual
         residual = x
-        x = ops.rmsnorm(x, fuse[0], fuse[1])
+        with _span(timer, "rmsnorm"):
+            x = ops.rmsnorm(x, fuse[0], fuse[1])
     cache = block.__dict__.setdefault("_moe_cache", {})
     gw = _gate_weight_bf16(gate_weight, cache)
     b = None if bias is None else bias.data.to(torch.float32)
-    timer = getattr(block, "stage_timer", None)
     with _span(timer, "router"):
         idx, w, logits = ops.router(x, gw, b, spec, want_logits)
     block.last_topk_idx, block.last_topk_weight = idx, w
