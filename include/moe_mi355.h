@@ -277,6 +277,50 @@ int moe_stage_stats(moe_stager* s, int64_t* n_copies, int64_t* n_bytes);
 int moe_stage_sync(moe_stager* s);
 int moe_stage_destroy(moe_stager* s);
 
+/* ------------------------------------------------- weight arena index (wire format) */
+
+/*
+ * Where each module's tensors lie inside one contiguous host arena: the reference's
+ * map module_key -> tensor_key -> tensor_meta{offset, tensor_shape, byte_size}
+ * (core/Parameter_Server/Parameter_Server.h:48-59) and its length-prefixed serialisation
+ * (compute_serialized_size / serialize_map_to_buffer / deserialize_map_from_buffer,
+ * core/Parameter_Server/posix_shm.cpp:167-357), byte-compatible on the wire:
+ *   u64 n_modules { u64 len, key, u64 n_tensors { u64 len, key, i64 offset, i64 byte_size,
+ *   u64 ndim, i64 shape[ndim] } }      (native endian, no padding)
+ * Parse errors carry the reference's "Buffer overflow (reading ...)" messages.
+ */
+typedef struct moe_arena_index moe_arena_index;
+
+int moe_arena_index_create(moe_arena_index** out);
+int moe_arena_index_destroy(moe_arena_index* ix);
+/* Insert or overwrite one tensor entry; modules and tensors keep insertion order. */
+int moe_arena_index_add(moe_arena_index* ix, const char* module_key, const char* tensor_key,
+                        int64_t offset, int64_t byte_size, const int64_t* shape, int32_t ndim);
+/* deserialize_map_from_buffer (posix_shm.cpp:270-357). */
+int moe_arena_index_parse(const void* buf, size_t bytes, moe_arena_index** out);
+/* compute_serialized_size (posix_shm.cpp:167-190). */
+size_t moe_arena_index_wire_size(const moe_arena_index* ix);
+/* serialize_map_to_buffer (posix_shm.cpp:196-268); capacity must be >= the wire size. */
+int moe_arena_index_serialize(const moe_arena_index* ix, void* buf, size_t capacity);
+int32_t moe_arena_index_n_modules(const moe_arena_index* ix);
+/* Key and tensor count of module i; pointers stay valid until the index changes. */
+int moe_arena_index_module(const moe_arena_index* ix, int32_t i, const char** key, int32_t* n_tensors);
+/* Position of a module key, or -1. */
+int moe_arena_index_find(const moe_arena_index* ix, const char* module_key);
+int moe_arena_index_tensor(const moe_arena_index* ix, int32_t i, int32_t j, const char** key,
+                           int64_t* offset, int64_t* byte_size, int32_t* ndim, const int64_t** shape);
+/*
+ * Register module `module_key` with a stager, its tensors read from arena_base + offset
+ * (Weights_Storage::Init, core/Weights_Storage/Weights_Storage.cpp:52-77; a missing key fails
+ * with "Module key not found in storage" as :80-87 does).  tensor_keys[i] is copied to
+ * dst_offsets[i] of the slot.  The arena must be pinned host memory that was ALLOCATED pinned;
+ * this library never registers existing memory.  Returns the module id (>= 0).
+ */
+int moe_stage_add_module_from_arena(moe_stager* s, int32_t type, const moe_arena_index* ix,
+                                    const char* module_key, const void* arena_base,
+                                    size_t arena_bytes, int32_t n_tensors,
+                                    const char* const* tensor_keys, const size_t* dst_offsets);
+
 #ifdef __cplusplus
 }
 #endif

@@ -47,6 +47,23 @@ SIGNATURES = {
     "moe_combine_residual": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32,
                                             c_int32, c_int32, c_int32, c_void_p, c_void_p]),
     "moe_rmsnorm": (ctypes.c_int, [c_void_p, c_void_p, ctypes.c_float, c_int32, c_int32, c_void_p, c_void_p]),
+    "moe_arena_index_create": (ctypes.c_int, [ctypes.POINTER(c_void_p)]),
+    "moe_arena_index_destroy": (ctypes.c_int, [c_void_p]),
+    "moe_arena_index_add": (ctypes.c_int, [c_void_p, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int64, ctypes.c_int64,
+                                           ctypes.POINTER(ctypes.c_int64), c_int32]),
+    "moe_arena_index_parse": (ctypes.c_int, [c_void_p, c_size_t, ctypes.POINTER(c_void_p)]),
+    "moe_arena_index_wire_size": (c_size_t, [c_void_p]),
+    "moe_arena_index_serialize": (ctypes.c_int, [c_void_p, c_void_p, c_size_t]),
+    "moe_arena_index_n_modules": (c_int32, [c_void_p]),
+    "moe_arena_index_module": (ctypes.c_int, [c_void_p, c_int32, ctypes.POINTER(ctypes.c_char_p),
+                                              ctypes.POINTER(c_int32)]),
+    "moe_arena_index_find": (ctypes.c_int, [c_void_p, ctypes.c_char_p]),
+    "moe_arena_index_tensor": (ctypes.c_int, [c_void_p, c_int32, c_int32, ctypes.POINTER(ctypes.c_char_p),
+                                              ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64),
+                                              ctypes.POINTER(c_int32), ctypes.POINTER(ctypes.POINTER(ctypes.c_int64))]),
+    "moe_stage_add_module_from_arena": (ctypes.c_int, [c_void_p, c_int32, c_void_p, ctypes.c_char_p, c_void_p, c_size_t,
+                                                       c_int32, ctypes.POINTER(ctypes.c_char_p),
+                                                       ctypes.POINTER(c_size_t)]),
     "moe_stage_create": (ctypes.c_int, [ctypes.POINTER(c_void_p), c_int32, ctypes.POINTER(c_size_t),
                                         ctypes.POINTER(c_int32), ctypes.POINTER(c_void_p), c_int32]),
     "moe_stage_set_policy": (ctypes.c_int, [c_void_p, c_int32, c_int32]),

@@ -113,6 +113,34 @@ class Stager:
         self.type_of[module_key] = module_type
         return mid
 
+    def add_module_from_arena(self, module_key: str, module_type: str, arena) -> int:
+        """Register `module_key` with its tensors read in place from an Arena (the reference's
+        Weights_Storage views into the shared weight segment, Weights_Storage.cpp:52-77)."""
+        lay = self.layout[module_type]
+        entries = arena.index.modules().get(module_key)
+        if entries is None:
+            raise RuntimeError(f"Module key not found in storage: {module_key}")
+        for name, (off, b, shape, dtype) in lay.items():
+            if name not in entries:
+                raise RuntimeError(f"module {module_key}: arena has no tensor {name}")
+            if entries[name][1] != b or tuple(entries[name][2]) != shape:
+                raise RuntimeError(f"module {module_key}.{name}: arena entry {entries[name][1:]} does not match "
+                                   f"the slot layout ({b} bytes, shape {shape})")
+        if self.backend == "device" and not arena.data.is_pinned():
+            raise RuntimeError("the arena must be pinned host memory (allocate it with pin_memory=True)")
+        n = len(lay)
+        keys = (ctypes.c_char_p * n)(*[k.encode() for k in lay])
+        offs = (ctypes.c_size_t * n)(*[v[0] for v in lay.values()])
+        mid = N.lib().moe_stage_add_module_from_arena(self._h, self.types.index(module_type), arena.index._h,
+                                                      module_key.encode(), arena.data.data_ptr(), arena.data.numel(),
+                                                      n, keys, offs)
+        if mid < 0:
+            N.check(mid, "moe_stage_add_module_from_arena")
+        self._src.append(arena)
+        self.ids[module_key] = mid
+        self.type_of[module_key] = module_type
+        return mid
+
     def set_policy(self, module_type: str, policy: str) -> None:
         """"cyclic": every module of the type is copied in registration order whether or not it
         will be used (the reference's worker, HtoD_Engine.cpp:201-268); "on_demand": only the

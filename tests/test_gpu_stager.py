@@ -188,3 +188,28 @@ def test_block_with_routing_aware_staging():
         assert st.stats()[0] - c0 == used + 1, (rep, st.stats()[0] - c0, used)   # + the shared expert
         assert not any(st.resident(f"routed_expert_{L}_{e}") for e in range(w.E))
     st.close()
+
+
+def test_arena_to_hbm():
+    """Modules registered from a pinned arena through its wire-format index arrive byte for byte."""
+    from moe_gen_amd import Arena, Stager
+    shapes = {"routed_expert": {"gate_proj.weight": ((64, 128), torch.float8_e4m3fn),
+                                "up_proj.weight": ((64, 128), torch.float8_e4m3fn),
+                                "down_proj.weight": ((128, 64), torch.float8_e4m3fn)}}
+    g = torch.Generator().manual_seed(1)
+    mods = {f"routed_expert_2_{e}": {n: torch.randint(0, 255, s, generator=g, dtype=torch.uint8).view(d)
+                                     for n, (s, d) in shapes["routed_expert"].items()} for e in range(6)}
+    packed = Arena.pack(mods)
+    arena = Arena.from_bytes(packed.index.serialize(), packed.data)       # what a second process would do
+    assert arena.data.is_pinned()
+    st = Stager(shapes, {"routed_expert": 3}, model_type="deepseek_v3", num_hidden_layers=4, num_local_experts=6)
+    for mk in mods:
+        st.add_module_from_arena(mk, "routed_expert", arena)
+    for rep in range(2):
+        for mk, tensors in mods.items():
+            w = st.get_weights(mk)
+            torch.cuda.synchronize()
+            for n, t in tensors.items():
+                assert torch.equal(w[n].view(torch.uint8).cpu(), t.view(torch.uint8)), (mk, n)
+            st.free_weights_buffer(mk)
+    st.close()
