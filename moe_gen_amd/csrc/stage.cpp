@@ -173,6 +173,7 @@ extern "C" int moe_stage_create(moe_stager** out, int32_t n_types, const size_t*
                 e = hipEventCreateWithFlags(&t.freed[s], hipEventDisableTiming);
                 if (e != hipSuccess) {
                     moe::set_error("moe_stage_create: hipEventCreateWithFlags: %s", hipGetErrorString(e));
+                    moe_stage_destroy(st);   // releases the stream and the events made so far
                     return MOE_ERR_HIP;
                 }
             }
