@@ -240,7 +240,7 @@ def run_workload(name: str, args, with_cpu: bool):
     gemm_tflops = (w.routed_flop + w.shared_flop) / (gemm_ms * 1e-3) / 1e12
     disp_bytes = w.dispatch_bytes if args.materialize else 4.0 * w.n * w.k
     mean_rows = w.n * w.k // w.E
-    mt = 4 if mean_rows >= 192 else (2 if mean_rows >= 96 else 1)
+    mt = 4 if mean_rows >= 192 else (2 if mean_rows >= 48 else 1)
     wbytes = 3.0 * w.E * w.h * w.I * (1 if w.fp8 else 2)
     result = {
         "metric": "MoE-layer tokens/sec at DeepSeek-V3 W8A16 shape" if name == "deepseek_v3_w8a16"
