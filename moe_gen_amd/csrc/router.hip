@@ -418,7 +418,12 @@ extern "C" int moe_router(const void* x, const void* w_gate, const float* bias, 
     if (E <= 32) return few ? launch<false, 1, 1, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st)
                             : launch<false, 1, 1, 4>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
     if (E <= 64) return launch<false, 1, 2, 2>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    if (E <= 128) return launch<false, 2, 2, 2>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    if (E <= 192) return launch<false, 2, 3, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    return launch<false, 2, 4, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    // more than 64 experts: one wave per 32 experts (one MFMA per k and wave, no padding beyond
+    // the next multiple of 32) measured 10-25 % faster than half as many waves with two MFMAs each
+    if (E <= 96) return launch<false, 1, 3, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    if (E <= 128) return launch<false, 1, 4, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    if (E <= 160) return launch<false, 1, 5, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    if (E <= 192) return launch<false, 1, 6, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    if (E <= 224) return launch<false, 1, 7, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    return launch<false, 1, 8, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
 }

@@ -119,3 +119,28 @@ def test_router_and_dispatch_golden_fixtures():
         counts, offsets, perm, pos, _ = ops.dispatch(torch.from_numpy(idx).cuda(), spec.n_experts)
         assert np.array_equal(counts.cpu().numpy(), z["counts"]) and np.array_equal(perm.cpu().numpy(), z["perm"])
         assert np.array_equal(offsets.cpu().numpy(), z["offsets"]) and np.array_equal(pos.cpu().numpy(), z["pos"])
+
+
+@pytest.mark.parametrize("E", [2, 4, 5, 8, 12, 16, 17, 32, 33, 64, 65, 96, 100, 128, 144, 160, 176, 192, 200, 224,
+                               250, 256])
+def test_every_expert_count_bracket(E):
+    """One case per kernel instantiation (and an odd count inside it): greedy softmax routing and,
+    where the count allows groups, sigmoid group-limited routing; logits, indices and weights
+    bit-for-bit.  n = 150 covers two full 64-token tiles and a ragged one; n = 16500 takes the
+    many-token instantiation of the E <= 32 bracket."""
+    print(f"router bracket E={E}", flush=True)
+    k = min(6, E)
+    g = torch.Generator().manual_seed(E)
+    specs = [(O.RouterSpec.deepseek_v2(E, k, "greedy", scale=1.0), False)]
+    if E % 4 == 0 and E >= 16:
+        specs.append((O.RouterSpec.deepseek_v3(E, k, 4, 2, True, 2.5), True))
+    for n, h in ((150, 136), (16500, 16)) if E in (17, 32) else ((150, 136),):
+        x = torch.randn(n, h, generator=g).to(torch.bfloat16)
+        wg = (torch.randn(E, h, generator=g) * 0.1).to(torch.bfloat16)
+        for spec, has_bias in specs:
+            bias = (torch.randn(E, generator=g) * 0.01) if has_bias else None
+            idx, w, lg = gpu_router(x, wg, bias, spec)
+            oi, ow, ol = O.router(bits(x), bits(wg), None if bias is None else bias.numpy(), spec)
+            assert np.array_equal(lg.view(np.uint32), ol.view(np.uint32)), (E, n, spec.method)
+            assert np.array_equal(idx, oi), (E, n, spec.method)
+            assert np.array_equal(w.view(np.uint32), ow.view(np.uint32)), (E, n, spec.method)
