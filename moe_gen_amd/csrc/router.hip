@@ -20,6 +20,8 @@
 // (lane l holds experts l, l+64, l+128, l+192) and wave-level butterfly
 // reductions.  Ties go to the lower expert (group) index and the slot order of
 // the output is the selection order (descending score).
+#include <type_traits>
+
 #include "common.h"
 #include "moe_math.h"
 
@@ -34,34 +36,68 @@ struct ArgMax {
     int i;
 };
 
+// Value held by the lane's xor-M partner, without going through LDS: cross-row exchanges with
+// the gfx950 lane-swap instructions, inside a 16-lane row with DPP.  M = 4 uses a rotation by 4,
+// which delivers the xor-4 partner's VALUE whenever the data already agrees between lanes l and
+// l^8 -- true in every butterfly below, where the step for 8 precedes the step for 4.
+template <int M>
+__device__ __forceinline__ int partner_bits(int x) {
+    const int lane = threadIdx.x & 63;
+    if constexpr (M == 32) {
+        auto r = __builtin_amdgcn_permlane32_swap(x, x, false, false);   // r[0] = low half twice, r[1] = high half twice
+        return (lane & 32) ? (int)r[0] : (int)r[1];
+    } else if constexpr (M == 16) {
+        auto r = __builtin_amdgcn_permlane16_swap(x, x, false, false);   // r[0] = even rows twice, r[1] = odd rows twice
+        return (lane & 16) ? (int)r[0] : (int)r[1];
+    } else if constexpr (M == 8) {
+        return __builtin_amdgcn_update_dpp(x, x, 0x128, 0xf, 0xf, false);   // row_ror:8
+    } else if constexpr (M == 4) {
+        return __builtin_amdgcn_update_dpp(x, x, 0x124, 0xf, 0xf, false);   // row_ror:4
+    } else if constexpr (M == 2) {
+        return __builtin_amdgcn_update_dpp(x, x, 0x4E, 0xf, 0xf, false);    // quad_perm [2,3,0,1]
+    } else {
+        return __builtin_amdgcn_update_dpp(x, x, 0xB1, 0xf, 0xf, false);    // quad_perm [1,0,3,2]
+    }
+}
+template <int M>
+__device__ __forceinline__ float partner(float v) {
+    return __builtin_bit_cast(float, partner_bits<M>(__builtin_bit_cast(int, v)));
+}
+
+template <int GW, int M = GW / 2, typename F>
+__device__ __forceinline__ void butterfly(F&& step) {
+    if constexpr (M >= 1) {
+        step(std::integral_constant<int, M>{});
+        butterfly<GW, M / 2>(step);
+    }
+}
+
 // max by value, equal values -> lower index
 template <int GW>
 __device__ __forceinline__ ArgMax group_argmax(ArgMax a) {
-#pragma unroll
-    for (int m = GW / 2; m >= 1; m >>= 1) {
-        float ov = __shfl_xor(a.v, m);
-        int oi = __shfl_xor(a.i, m);
-        bool take = (ov > a.v) || (ov == a.v && oi < a.i);
+    butterfly<GW>([&](auto m) {
+        const float ov = partner<decltype(m)::value>(a.v);
+        const int oi = partner_bits<decltype(m)::value>(a.i);
+        const bool take = (ov > a.v) || (ov == a.v && oi < a.i);
         a.v = take ? ov : a.v;
         a.i = take ? oi : a.i;
-    }
+    });
     return a;
 }
 
 template <int GW>
 __device__ __forceinline__ float group_max(float v) {
-#pragma unroll
-    for (int m = GW / 2; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m));
+    butterfly<GW>([&](auto m) { v = fmaxf(v, partner<decltype(m)::value>(v)); });
     return v;
 }
 
 // The canonical sum over experts: 64 strided partials folded by the butterfly 32,16,8,4,2,1
-// (p[l] += p[l^m]; fp32 addition commutes).  With E <= 16 the partials of lanes 16..63 are +0, the
-// steps 32 and 16 add +0 to non-negative values, and the remaining steps are the 16-lane butterfly.
+// (p[l] += p[l^m]; fp32 addition commutes).  With E <= 16 (E <= 32) the partials of lanes 16..63
+// (32..63) are +0, the leading steps add +0 to non-negative values, and the remaining steps are the
+// 16-lane (32-lane) butterfly.
 template <int GW>
 __device__ __forceinline__ float group_sum_butterfly(float v) {
-#pragma unroll
-    for (int m = GW / 2; m >= 1; m >>= 1) v = v + __shfl_xor(v, m);
+    butterfly<GW>([&](auto m) { v = v + partner<decltype(m)::value>(v); });
     return v;
 }
 
@@ -70,11 +106,11 @@ constexpr int kBigIdx = 0x7fffffff;
 
 // Routes one token per lane group; `row` points at the group's logits (LDS, E valid entries).
 // `live` is false for groups without a token (they run the same code on a valid row, store nothing).
-template <int GW>
+template <int GW, int MAX_EJ>
 __device__ void route_token(const float* row, const float* __restrict__ bias, const moe_router_params& p,
                             int32_t* __restrict__ idx_out, float* __restrict__ w_out,
                             float* __restrict__ logits_out, bool live) {
-    constexpr int MAX_EJ = GW == 64 ? 4 : 1;   // experts per lane (E <= 256, or E <= 16)
+    // MAX_EJ: experts per lane, ceil(padded experts / GW)
     const int lane = threadIdx.x & 63, gl = lane & (GW - 1), gbase = lane - gl;
     const int E = p.n_experts;
     float L[MAX_EJ], s[MAX_EJ], c[MAX_EJ];
@@ -227,20 +263,24 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     const int t0 = blockIdx.x * BT;
 
     u32x4 xr[2][XPT], wr[2][WPT];
+    // Loads are unconditional (addresses clamped; chunks beyond h are zeroed when they are stored
+    // to LDS, two stages later): a load under a branch makes the compiler wait for ALL outstanding
+    // loads before the first LDS store of a stage, and a select right after the load makes it
+    // wait at once; either would undo the two-stage prefetch.
     auto load_stage = [&](int k0, int set) {
 #pragma unroll
         for (int i = 0; i < XPT; ++i) {
-            int c = tid + i * NT;
-            int row = c / (KC / 8), kk = k0 + (c % (KC / 8)) * 8;
-            int t = min(t0 + row, n - 1);
-            xr[set][i] = (c < XCH && kk < h) ? *reinterpret_cast<const u32x4*>(x + (size_t)t * h + kk) : u32x4{0, 0, 0, 0};
+            const int c = tid + i * NT;
+            const int row = c / (KC / 8), kk = k0 + (c % (KC / 8)) * 8;
+            const int t = min(t0 + row, n - 1);
+            xr[set][i] = *reinterpret_cast<const u32x4*>(x + (size_t)t * h + (kk < h ? kk : 0));
         }
 #pragma unroll
         for (int i = 0; i < WPT; ++i) {
-            int c = tid + i * NT;
-            int row = c / (KC / 8), kk = k0 + (c % (KC / 8)) * 8;
-            int e = min(row, E - 1);
-            wr[set][i] = (c < WCH && kk < h) ? *reinterpret_cast<const u32x4*>(wg + (size_t)e * h + kk) : u32x4{0, 0, 0, 0};
+            const int c = tid + i * NT;
+            const int row = c / (KC / 8), kk = k0 + (c % (KC / 8)) * 8;
+            const int e = min(row, E - 1);
+            wr[set][i] = *reinterpret_cast<const u32x4*>(wg + (size_t)e * h + (kk < h ? kk : 0));
         }
     };
     auto store_chunk = [&](float* base, int c, u32x4 v) {
@@ -253,16 +293,18 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
         *reinterpret_cast<f32x4*>(d) = lo;
         *reinterpret_cast<f32x4*>(d + 4) = hi;
     };
-    auto store_stage = [&](int set) {
+    auto store_stage = [&](int set, int k0) {
 #pragma unroll
         for (int i = 0; i < XPT; ++i) {
             int c = tid + i * NT;
-            if (c < XCH) store_chunk(Xs, c, xr[set][i]);
+            const bool ok = k0 + (c % (KC / 8)) * 8 < h;
+            if (c < XCH) store_chunk(Xs, c, ok ? xr[set][i] : u32x4{0, 0, 0, 0});
         }
 #pragma unroll
         for (int i = 0; i < WPT; ++i) {
             int c = tid + i * NT;
-            if (c < WCH) store_chunk(Ws, c, wr[set][i]);
+            const bool ok = k0 + (c % (KC / 8)) * 8 < h;
+            if (c < WCH) store_chunk(Ws, c, ok ? wr[set][i] : u32x4{0, 0, 0, 0});
         }
     };
 
@@ -309,13 +351,16 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
         }
     };
 
+    // No load sits under a branch (the tail re-loads the last stage instead of skipping): with
+    // straight-line code the compiler counts outstanding loads exactly and a stage waits only for
+    // the register set it stores, not for the set that was requested one stage ago.
     const int nstage = (h + KC - 1) / KC;
     load_stage(0, 0);
-    if (nstage > 1) load_stage(KC, 1);
+    load_stage(min(1, nstage - 1) * KC, 1);
     auto stage = [&](int st, int set) {      // set == st & 1, a literal at both call sites
-        store_stage(set);
+        store_stage(set, st * KC);
         __syncthreads();
-        if (st + 2 < nstage) load_stage((st + 2) * KC, set);
+        load_stage(min(st + 2, nstage - 1) * KC, set);
         multiply_stage();
         __syncthreads();
     };
@@ -355,15 +400,17 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     }
     __syncthreads();
 
-    // selection: a lane group per token (4 tokens per wave at a time when E <= 16)
-    constexpr int NW = WE * WT, GW = SMALL ? 16 : 64, TPW = 64 / GW;
+    // selection, a lane group per token: 16 lanes for E <= 16, 32 for E <= 32, else the whole wave with
+    // ceil(EP / 64) experts per lane
+    constexpr int NW = WE * WT, GW = SMALL ? 16 : (EP <= 32 ? 32 : 64), TPW = 64 / GW;
+    constexpr int EJ = (EP + GW - 1) / GW;
     for (int tb = wave * TPW; tb < BT; tb += NW * TPW) {
         if (t0 + tb >= n) break;
         const int tl = tb + (lane / GW);
         const int t = t0 + tl;
         const bool live = t < n;
         const int tr = live ? t : n - 1, tlr = live ? tl : tb;
-        route_token<GW>(lg + tlr * EP, bias, p, topk_idx + (size_t)tr * p.top_k, topk_w + (size_t)tr * p.top_k,
+        route_token<GW, EJ>(lg + tlr * EP, bias, p, topk_idx + (size_t)tr * p.top_k, topk_w + (size_t)tr * p.top_k,
                         logits_out ? logits_out + (size_t)tr * E : nullptr, live);
     }
 }
