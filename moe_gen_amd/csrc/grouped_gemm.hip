@@ -340,31 +340,47 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     const int nk = K / BK;
     gload(0, 0);
     lds_store(smem0, 0);
+    // No load or store of the pipeline sits under a branch (past the end the last tile is loaded
+    // again and stored where nobody reads it): with straight-line code the compiler counts the
+    // outstanding loads exactly, so storing register set d waits for set d only, not for the set
+    // requested an iteration later -- under a branch it waits for everything and PF = 2 buys nothing.
 #pragma unroll
-    for (int d = 0; d < PF; ++d)
-        if (1 + d < nk) gload(1 + d, d);
+    for (int d = 0; d < PF; ++d) gload(min(1 + d, nk - 1), d);
     __syncthreads();
+    // The two waves of a SIMD run the MFMA half and the data half of an iteration in opposite
+    // order: waves 0-3 multiply tile kt and then move data, waves 4-7 move data first.  Both kinds
+    // share ONE copy of the data half: the loop body is "store, load, [barrier,] multiply
+    // [, barrier]", in which waves 0-3 multiply the NEXT tile after the barrier (their first tile is
+    // multiplied ahead of the loop) and waves 4-7 multiply the current tile before it.  Every wave
+    // still passes one barrier per iteration, and no global load sits inside a region that only
+    // some waves execute -- there the compiler must assume the loads were never issued and makes
+    // each LDS store wait for all outstanding loads, which silently undoes the second register set.
     const bool mfma_first = wave < 4;   // waves w and w+4 share a SIMD
+    if (mfma_first) {
+        __builtin_amdgcn_s_setprio(2);
+        compute(smem0, false);
+        __builtin_amdgcn_s_setprio(0);
+    }
     // iteration kt: tile kt+1 is in register set kt % PF; it moves to the other LDS stage and the
     // set is refilled with tile kt+1+PF (the loop is unrolled by PF so the set index is static)
     auto iteration = [&](int kt, int set) {
         const uint8_t* rd = (kt & 1) ? smem1 : smem0;
         uint8_t* wr = (kt & 1) ? smem0 : smem1;
-        // the wave that is multiplying outranks its SIMD partner that is moving data
+        lds_store(wr, set);
+        gload(min(kt + 1 + PF, nk - 1), set);
         if (mfma_first) {
-            __builtin_amdgcn_s_setprio(2);
-            compute(rd, kt > 0);
-            __builtin_amdgcn_s_setprio(0);
-            if (kt + 1 < nk) lds_store(wr, set);
-            if (kt + 1 + PF < nk) gload(kt + 1 + PF, set);
+            __syncthreads();   // (waits for this wave's LDS reads and writes, then for the other waves)
+            if (kt + 1 < nk) {
+                __builtin_amdgcn_s_setprio(2);
+                compute(wr, true);
+                __builtin_amdgcn_s_setprio(0);
+            }
         } else {
-            if (kt + 1 < nk) lds_store(wr, set);
-            if (kt + 1 + PF < nk) gload(kt + 1 + PF, set);
             __builtin_amdgcn_s_setprio(2);
             compute(rd, kt > 0);
             __builtin_amdgcn_s_setprio(0);
+            __syncthreads();
         }
-        __syncthreads();   // (waits for this wave's LDS reads and writes, then for the other waves)
     };
     int kt = 0;
     for (; kt + PF <= nk; kt += PF) {
