@@ -100,9 +100,8 @@ __device__ __forceinline__ const uint8_t* uni_ptr(const void* p) {
 }
 
 // MT: 32-row MFMA tiles per wave along M (workgroup rows BM = 64*MT, 2 waves along M)
-// WN: waves along N; 4 -> 8 waves of up to 128x64 outputs, two per SIMD, which issue their MFMA
-//     half and their load/dequantise/store half of an iteration in opposite order, so that one
-//     feeds the matrix core while the other feeds LDS
+// WN: waves along N; 4 -> 8 waves of up to 128x64 outputs, two per SIMD; every wave interleaves
+//     its share of the load / dequantise / LDS-store work with its MFMAs, a piece per MFMA group
 template <int MT, int WN, bool SWIGLU, bool W8>
 __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     constexpr int NT = 128 * WN;                // threads
@@ -317,22 +316,6 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
             for (int j = 0; j < NJ; ++j)
                 acc[mi][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[s & 1][j], tf[s & 1][mi], acc[mi][j], 0, 0, 0);
     };
-    // multiplies k-steps 0 .. LAST-1 of the tile in `As`, preceded by the pending last k-step of the
-    // previous tile; leaves the fragments of k-step LAST in registers
-    auto compute = [&](const uint8_t* As, bool have_pending) {
-        read_frags(As, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        if (have_pending) mfmas(LAST);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int s = 0; s < LAST; ++s) {
-            read_frags(As, s + 1);
-            __builtin_amdgcn_sched_barrier(0);
-            mfmas(s);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    };
-
     // ---- main loop ----
     // On entry to iteration kt: LDS stage kt&1 holds tile kt and the registers hold tiles kt+1 ..
     // kt+PF (possibly still in flight).  The iteration moves tile kt+1 into the other LDS stage,
@@ -340,47 +323,87 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     const int nk = K / BK;
     gload(0, 0);
     lds_store(smem0, 0);
-    // No load or store of the pipeline sits under a branch (past the end the last tile is loaded
-    // again and stored where nobody reads it): with straight-line code the compiler counts the
-    // outstanding loads exactly, so storing register set d waits for set d only, not for the set
-    // requested an iteration later -- under a branch it waits for everything and PF = 2 buys nothing.
+    // No load or store of the pipeline sits under a branch or in a region that only some waves
+    // execute (past the end the last tile is loaded again and stored where nobody reads it): with
+    // straight-line code the compiler counts the outstanding loads exactly, so a store waits only
+    // for the chunk it stores.  Under a branch it must assume the load may never have been issued
+    // and waits for ALL outstanding loads, which serialises the whole pipeline.
 #pragma unroll
     for (int d = 0; d < PF; ++d) gload(min(1 + d, nk - 1), d);
     __syncthreads();
-    // The two waves of a SIMD run the MFMA half and the data half of an iteration in opposite
-    // order: waves 0-3 multiply tile kt and then move data, waves 4-7 move data first.  Both kinds
-    // share ONE copy of the data half: the loop body is "store, load, [barrier,] multiply
-    // [, barrier]", in which waves 0-3 multiply the NEXT tile after the barrier (their first tile is
-    // multiplied ahead of the loop) and waves 4-7 multiply the current tile before it.  Every wave
-    // still passes one barrier per iteration, and no global load sits inside a region that only
-    // some waves execute -- there the compiler must assume the loads were never issued and makes
-    // each LDS store wait for all outstanding loads, which silently undoes the second register set.
-    const bool mfma_first = wave < 4;   // waves w and w+4 share a SIMD
-    if (mfma_first) {
-        __builtin_amdgcn_s_setprio(2);
-        compute(smem0, false);
-        __builtin_amdgcn_s_setprio(0);
-    }
-    // iteration kt: tile kt+1 is in register set kt % PF; it moves to the other LDS stage and the
-    // set is refilled with tile kt+1+PF (the loop is unrolled by PF so the set index is static)
+    // One data item = one LDS store's worth of this thread's staged chunks (a 16-byte token chunk,
+    // a 16-byte bf16 weight chunk, or half of a 16-byte fp8 weight chunk -> 8 bf16): store it to the
+    // other stage and, once a chunk's last item is stored, refill its registers with the chunk of
+    // tile kt+1+PF.  The items are spread over the iteration, one per group of MFMAs, so LDS, the
+    // vector-memory pipe and the matrix core see a steady mix instead of bursts; with exact load
+    // waits each item stalls only until its own chunk (requested PF iterations earlier) is there.
+    constexpr int NBI = W8 ? 2 * NB : NB;
+    constexpr int NI = NA + NBI;
+    auto data_item = [&](int i, uint8_t* As, int kt, int set) {
+        uint8_t* Bs = As + A_STAGE;
+        const int kn = min(kt + 1 + PF, nk - 1);
+        const size_t kofs = (size_t)kn * BK;
+        if (i < NA) {
+            *reinterpret_cast<u32x4*>(As + a_lds + i * RA * ROW_B) = ra[set][i];
+            ra[set][i] = gload16(g.a + (size_t)a_src[i] * K + kofs + lchunk * 8);
+        } else if (W8) {
+            const int b = (i - NA) >> 1, half = (i - NA) & 1;
+            const uint8_t* m = (SWIGLU && b >= NB / 2) ? bmat1 : bmat0;
+            const float sc = rs[set][b / (NB / 2)];
+            const uint32_t q0 = rb[set][b][2 * half], q1 = rb[set][b][2 * half + 1];
+            const f32x2 c0 = __builtin_amdgcn_cvt_pk_f32_fp8(q0, false), c1 = __builtin_amdgcn_cvt_pk_f32_fp8(q0, true);
+            const f32x2 c2 = __builtin_amdgcn_cvt_pk_f32_fp8(q1, false), c3 = __builtin_amdgcn_cvt_pk_f32_fp8(q1, true);
+            const u32x4 o = {pack_bf16(c0[0] * sc, c0[1] * sc), pack_bf16(c1[0] * sc, c1[1] * sc),
+                             pack_bf16(c2[0] * sc, c2[1] * sc), pack_bf16(c3[0] * sc, c3[1] * sc)};
+            // the first 8 weights go to b_lds[0], the second 8 to b_lds[1]; swapped rows the other way round
+            *reinterpret_cast<u32x4*>(Bs + ((half ^ (b_swap ? 1 : 0)) ? b_lds[1] : b_lds[0]) + b * RB * ROW_B) = o;
+            if (half == 1) {
+                rb[set][b] = gload16(m + ((size_t)b_n[b] * K + kofs) * EB + bcol_b);
+                if (b / (NB / 2) == 0) rs[set][0] = sc0[srow0 + (kn >> 1)];
+                else rs[set][1] = sc1[srow1 + (kn >> 1)];
+            }
+        } else {
+            const int b = i - NA;
+            const uint8_t* m = (SWIGLU && b >= NB / 2) ? bmat1 : bmat0;
+            *reinterpret_cast<u32x4*>(Bs + b_lds[0] + b * RB * ROW_B) = rb[set][b];
+            rb[set][b] = gload16(m + ((size_t)b_n[b] * K + kofs) * EB + bcol_b);
+        }
+    };
+    constexpr int MPS = MT * NJ;                  // MFMAs per k-step
+    constexpr int GPS = MPS >= 8 ? 2 : 1;         // MFMA groups per k-step
+    constexpr int MPG = MPS / GPS, NG = NS * GPS; // MFMAs per group, groups per iteration
+    auto mfma_group = [&](int s, int gg) {
+#pragma unroll
+        for (int m = gg * MPG; m < (gg + 1) * MPG; ++m) {
+            const int mi = m / NJ, j = m % NJ;
+            acc[mi][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[s & 1][j], tf[s & 1][mi], acc[mi][j], 0, 0, 0);
+        }
+    };
+    // iteration kt multiplies tile kt out of stage kt&1 (the MFMAs of its k-step t are issued one
+    // step late, behind the fragment reads of step t+1; those of its last step behind the first
+    // reads of the next tile, across the barrier) while tile kt+1 moves from register set kt % PF
+    // (the loop is unrolled by PF so the set index is static) into the other stage.
     auto iteration = [&](int kt, int set) {
         const uint8_t* rd = (kt & 1) ? smem1 : smem0;
         uint8_t* wr = (kt & 1) ? smem0 : smem1;
-        lds_store(wr, set);
-        gload(min(kt + 1 + PF, nk - 1), set);
-        if (mfma_first) {
-            __syncthreads();   // (waits for this wave's LDS reads and writes, then for the other waves)
-            if (kt + 1 < nk) {
-                __builtin_amdgcn_s_setprio(2);
-                compute(wr, true);
-                __builtin_amdgcn_s_setprio(0);
+#pragma unroll
+        for (int t = 0; t < NS; ++t) {
+            read_frags(rd, t);
+#pragma unroll
+            for (int gg = 0; gg < GPS; ++gg) {
+                // group g takes items [g*NI/NG, (g+1)*NI/NG): in order, so the two halves of an fp8
+                // chunk are stored before its registers are refilled
+                const int grp = t * GPS + gg;
+#pragma unroll
+                for (int i = grp * NI / NG; i < (grp + 1) * NI / NG; ++i) data_item(i, wr, kt, set);
+                // fp8: the conversion of an item may be scheduled in between the MFMAs of its group
+                if (!W8) __builtin_amdgcn_sched_barrier(0);
+                if (t > 0) mfma_group(t - 1, gg);
+                else if (kt > 0) mfma_group(LAST, gg);
+                __builtin_amdgcn_sched_barrier(0);
             }
-        } else {
-            __builtin_amdgcn_s_setprio(2);
-            compute(rd, kt > 0);
-            __builtin_amdgcn_s_setprio(0);
-            __syncthreads();
         }
+        __syncthreads();   // (waits for this wave's LDS reads and writes, then for the other waves)
     };
     int kt = 0;
     for (; kt + PF <= nk; kt += PF) {

@@ -74,6 +74,9 @@ def run_case(E, h, I, counts, fp8, seed, use_row_map=False):
     (4, 256, 384, [0, 1, 255, 257]),
     (8, 512, 256, [5, 0, 130, 64, 0, 0, 700, 31]),
     (3, 1024, 640, [1000, 3, 500]),
+    (8, 256, 256, [3, 0, 40, 17, 0, 1, 64, 9]),        # mean < 48 rows per expert: the 64-row tile
+    (6, 384, 128, [70, 2, 0, 33, 1, 5]),
+    (2, 128, 128, [1, 0]),
 ])
 def test_grouped_swiglu_vs_oracle(fp8, E, h, I, counts):
     print(f"grouped fp8={fp8} E={E} h={h} I={I} counts={counts}", flush=True)
