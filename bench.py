@@ -294,7 +294,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--staged", action="store_true", help="also time the block with weights staged from pinned host memory")
     ap.add_argument("--decoder-half", action="store_true", help="also time RMSNorm + block + residual add, fused and separate")
-    ap.add_argument("--cpu-sample", type=int, default=256, help="tokens of the workload the CPU baseline runs")
+    ap.add_argument("--cpu-sample", type=int, default=1024, help="tokens of the workload the CPU baseline runs")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); use --gpus 1")

@@ -395,7 +395,12 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
                 // chunk are stored before its registers are refilled
                 const int grp = t * GPS + gg;
 #pragma unroll
-                for (int i = grp * NI / NG; i < (grp + 1) * NI / NG; ++i) data_item(i, wr, kt, set);
+                for (int i0 = grp * NI / NG; i0 < (grp + 1) * NI / NG; ++i0) {
+                    // fp8, 4 + 4 items: token chunks and weight half-chunks alternate, so the
+                    // conversion work is spread evenly over the iteration (headline -3 %)
+                    const int i = (W8 && NA == 4 && NI == 8) ? ((i0 & 1) ? NA + (i0 >> 1) : (i0 >> 1)) : i0;
+                    data_item(i, wr, kt, set);
+                }
                 // fp8: the conversion of an item may be scheduled in between the MFMAs of its group
                 if (!W8) __builtin_amdgcn_sched_barrier(0);
                 if (t > 0) mfma_group(t - 1, gg);
