@@ -91,3 +91,31 @@ def test_dense_equivalence():
     y = blk(x).float()
     ref = blk.experts[0](x).float()
     assert rel_max(y.cpu().numpy(), ref.cpu().numpy()) <= TOL
+
+
+@pytest.mark.parametrize("name", ["deepseek_v3_w8a16", "deepseek_v2_lite", "mixtral_8x7b"])
+def test_block_edge_shapes(name):
+    """Empty batch, a single token, a non-contiguous view, a batch of identical tokens (every row
+    takes the same experts: k experts get everything, the rest nothing)."""
+    from moe_gen_amd import synthetic
+    w = synthetic.WORKLOADS[name].scaled(n=64, h=512, I=256, seq=64)
+    blk = synthetic.build_block(w, device="cuda", gen_device="cpu")
+    first = lambda r: r[0] if isinstance(r, tuple) else r
+    x = synthetic.hidden_states(w, "cpu").cuda()                      # [1, 64, 512]
+    full = first(blk(x)).clone()
+    # empty
+    out = first(blk(x[:, :0]))
+    assert out.shape == (1, 0, w.h)
+    # one token: same bits as that token inside the batch (rows are independent)
+    one = first(blk(x[:, 5:6].contiguous()))
+    assert torch.equal(one, full[:, 5:6])
+    # non-contiguous input
+    xt = torch.empty(w.h, 64, dtype=torch.bfloat16, device="cuda").t().unsqueeze(0)   # strides (1, 64)
+    xt.copy_(x)
+    assert not xt.is_contiguous() and torch.equal(first(blk(xt)), full)
+    # identical tokens
+    same = x[:, :1].expand(1, 64, w.h).contiguous()
+    out = first(blk(same))
+    torch.cuda.synchronize()
+    assert int((blk.last_counts > 0).sum()) == w.k and int(blk.last_counts.max()) == 64
+    assert torch.equal(out, full[:, :1].expand_as(out))
