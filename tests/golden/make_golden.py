@@ -7,6 +7,7 @@ restatement (oracle/torch_blocks.py) wherever the scores have no near-ties.
 
     python tests/golden/make_golden.py
 """
+import json
 import os
 import sys
 
@@ -19,6 +20,7 @@ sys.path.insert(0, os.path.dirname(HERE))
 
 from oracle import oracle as O  # noqa: E402
 from oracle import torch_blocks as TB  # noqa: E402
+from oracle import arena_format as AF  # noqa: E402
 from util import bits  # noqa: E402
 
 
@@ -66,6 +68,29 @@ def main():
     s = (rng.random((2, 2)) * 0.02 + 1e-3).astype(np.float32)
     np.savez_compressed(os.path.join(HERE, "fp8_dequant.npz"), table=O.fp8_table(), q=q, scale=s,
                         out=O.dequant_block(q, s))
+    # RMSNorm (two row widths, one all-zero row, one large-magnitude row) and the residual add
+    g = torch.Generator().manual_seed(16)
+    for h in (64, 1544):
+        x = torch.randn(9, h, generator=g).to(torch.bfloat16)
+        x[0] = 0
+        x[1] *= 300
+        w = (1.0 + 0.2 * torch.randn(h, generator=g)).to(torch.bfloat16)
+        r = torch.randn(9, h, generator=g).to(torch.bfloat16)
+        out = O.rmsnorm(bits(x), bits(w), 1e-6)
+        witness = bits(w * (x.float() * torch.rsqrt(x.float().pow(2).mean(-1, keepdim=True) + 1e-6)).to(torch.bfloat16))
+        assert np.abs(out.astype(np.int32) - witness.astype(np.int32)).max() <= 1
+        np.savez_compressed(os.path.join(HERE, f"rmsnorm_{h}.npz"), x=bits(x), weight=bits(w), eps=np.float32(1e-6),
+                            out=out, residual=bits(r), out_plus_residual=O.add_residual(out, bits(r)))
+    # weight-arena index on the wire: three modules, ragged tensor lists, a 0-dim and a 4-dim shape
+    index = {"routed_expert_3_0": {"gate_proj.weight": (0, 29360128, (2048, 7168)),
+                                   "gate_proj.weight_scale_inv": (29360128, 3584, (16, 56))},
+             "shared_expert_3": {"down_proj.weight": (1 << 33, 12, (1, 2, 3, 2))},
+             "lm_head": {"scalar": (40, 4, ())}}
+    with open(os.path.join(HERE, "arena_index.bin"), "wb") as f:
+        f.write(AF.serialize(index))
+    with open(os.path.join(HERE, "arena_index.json"), "w") as f:
+        json.dump({mk: {tk: [o, nb, list(sh)] for tk, (o, nb, sh) in inner.items()} for mk, inner in index.items()}, f,
+                  indent=1)
 
 
 if __name__ == "__main__":

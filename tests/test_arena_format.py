@@ -125,3 +125,18 @@ def test_arena_feeds_the_stager():
     with pytest.raises(RuntimeError, match="does not match"):
         st.add_module_from_arena("routed_expert_0_1", "routed_expert", Arena(ix2, packed.data))
     st.close()
+
+
+def test_golden_wire_fixture():
+    """tests/golden/arena_index.bin against its JSON description: both parsers, and both writers
+    reproduce the bytes."""
+    import json
+    import os
+    here = os.path.join(os.path.dirname(__file__), "golden")
+    wire = open(os.path.join(here, "arena_index.bin"), "rb").read()
+    want = {mk: {tk: (o, nb, tuple(sh)) for tk, (o, nb, sh) in inner.items()}
+            for mk, inner in json.load(open(os.path.join(here, "arena_index.json"))).items()}
+    assert F.deserialize(wire) == want
+    ix = ArenaIndex.parse(wire)
+    assert ix.modules() == want and list(ix.modules()) == list(want)
+    assert ix.serialize() == wire and build(want).serialize() == wire and F.serialize(want) == wire

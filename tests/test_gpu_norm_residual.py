@@ -89,3 +89,24 @@ def test_fused_decoder_half_equals_composition(name):
     assert getattr(blk, "_norm_residual", None) is None      # a later plain call is the plain block
     again = blk(xn)
     assert torch.equal(again[0] if isinstance(again, tuple) else again, ref)
+
+
+def test_rmsnorm_golden_fixtures():
+    """The committed vectors (tests/golden/rmsnorm_*.npz) through the C ABI: the norm kernel, and the
+    residual add through the combine kernel with one slot of weight 1."""
+    import glob
+    import os
+    from moe_gen_amd import ops
+    from util import bf16_tensor
+    files = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "rmsnorm_*.npz")))
+    assert len(files) == 2
+    for f in files:
+        z = np.load(f)
+        x, w, r = (bf16_tensor(z[k]).cuda() for k in ("x", "weight", "residual"))
+        out = ops.rmsnorm(x, w, float(z["eps"]))
+        assert np.array_equal(bits(out), z["out"]), f
+        n = x.shape[0]
+        ident = torch.arange(n, dtype=torch.int32, device="cuda")
+        one = torch.ones(n, 1, device="cuda")
+        summed = ops.combine(out, ident, None, one, None, ops.COMBINE_F32, residual=r)
+        assert np.array_equal(bits(summed), z["out_plus_residual"]), f

@@ -68,3 +68,16 @@ def test_add_residual_is_torch_bf16_add():
     r = (torch.randn(50, 96, generator=g) * 50).to(torch.bfloat16)
     assert np.array_equal(O.add_residual(bits(a), bits(r)), bits(r + a))
     assert np.array_equal(O.add_residual(bits(a), bits(r)), O.add_residual(bits(r), bits(a)))
+
+
+def test_golden_fixtures():
+    """The committed vectors (tests/golden/rmsnorm_*.npz, written by tests/golden/make_golden.py)."""
+    import glob
+    import os
+    files = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "rmsnorm_*.npz")))
+    assert len(files) == 2
+    for f in files:
+        z = np.load(f)
+        out = O.rmsnorm(z["x"], z["weight"], float(z["eps"]))
+        assert np.array_equal(out, z["out"]), f
+        assert np.array_equal(O.add_residual(out, z["residual"]), z["out_plus_residual"]), f
