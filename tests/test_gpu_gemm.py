@@ -89,6 +89,31 @@ def test_grouped_swiglu_vs_oracle(fp8, E, h, I, counts):
 
 
 @pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("E,mean", [(700, 3), (1024, 2), (600, 200)])
+def test_grouped_many_experts(fp8, E, mean):
+    """More experts than threads in a workgroup (the M-tile prefix scan takes two passes), up to the
+    maximum of 1024, with empty experts sprinkled in; the last case takes the 256-row tile."""
+    print(f"grouped many experts fp8={fp8} E={E} mean={mean}", flush=True)
+    rng = np.random.default_rng(E)
+    counts = rng.poisson(mean, E)
+    counts[::7] = 0
+    y, ref32, _ = run_case(E, 128, 128, counts, fp8, seed=5)
+    assert np.isfinite(y).all() and rel_max(y, ref32) <= TOL
+
+
+def test_grouped_too_many_experts_is_an_error():
+    from moe_gen_amd import ops
+    E = 1025
+    w = torch.zeros(128, 128, dtype=torch.bfloat16, device="cuda")
+    ptrs = ops.expert_pointers([w] * E, [w] * E, [w] * E)
+    off = torch.zeros(E + 1, dtype=torch.int32, device="cuda")
+    off[1:] = 4
+    x = torch.zeros(4, 128, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError, match="n_experts"):
+        ops.grouped_swiglu(x, None, ptrs, off, 4)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
 def test_grouped_swiglu_row_map(fp8):
     y, ref32, _ = run_case(4, 256, 256, [100, 0, 300, 77], fp8, seed=23, use_row_map=True)
     assert rel_max(y, ref32) <= TOL
