@@ -20,18 +20,20 @@
 // so that each XCD owns a contiguous range of tiles (same expert, neighbouring M/N
 // tiles), which is what makes its private L2 hold the A and B panels that are re-read.
 //
-// Workgroup = 8 waves (2 along M, 4 along N), two per SIMD.  Per wave MT x 2 MFMA tiles of
-// 32x32 (v_mfma_f32_32x32x16_bf16), i.e. up to 128x64 outputs and 128 fp32 accumulators.
+// Workgroup = 8 waves (2 along M, 4 along N), two per SIMD.  Per wave 2*MT x 4 MFMA tiles of
+// 16x16 (v_mfma_f32_16x16x32_bf16), i.e. up to 128x64 outputs and 128 fp32 accumulators.  On
+// real (non-zero) data this chip is power-limited under MFMA load; the 16x16x32 shape moves a
+// third less accumulator data per flop than 32x32x16 and sustains ~13 % more (1.95 vs 1.73
+// PFLOP/s in a registers-only loop with random operands), which is worth ~6 % here.
 // K advances 64 at a time through two LDS stages; rows are 128 bytes with a 16-byte-chunk
 // XOR swizzle so that both the 16-byte stores and the 16-byte MFMA operand reads are
 // bank-conflict free.  Global loads for tile k+2 are in flight while tile k is multiplied
-// and tile k+1 is written to LDS.  The two waves of a SIMD run the halves of an iteration
-// (MFMA work / data movement) in opposite order, so the matrix core and the LDS port are
-// both kept busy between the one barrier per k-stage.
+// and tile k+1 is written to LDS; every wave interleaves its share of that data movement with
+// its MFMAs, one piece per group of MFMAs, between the one barrier per k-stage.
 //
 // The MFMA is issued with the WEIGHT fragment as srcA and the TOKEN fragment as srcB, so
-// a lane ends up holding 4 consecutive output columns of one token row per register
-// quad; the epilogue transposes them through LDS into 16-byte-per-lane row-contiguous stores.
+// a lane ends up holding 4 consecutive output columns of one token row per accumulator;
+// the epilogue transposes them through LDS into 16-byte-per-lane row-contiguous stores.
 
 #include "common.h"
 
@@ -99,7 +101,7 @@ __device__ __forceinline__ const uint8_t* uni_ptr(const void* p) {
     return reinterpret_cast<const uint8_t*>((uintptr_t)(((uint64_t)hi << 32) | lo));
 }
 
-// MT: 32-row MFMA tiles per wave along M (workgroup rows BM = 64*MT, 2 waves along M)
+// MT: 32-row units per wave along M (workgroup rows BM = 64*MT, 2 waves along M)
 // WN: waves along N; 4 -> 8 waves of up to 128x64 outputs, two per SIMD; every wave interleaves
 //     its share of the load / dequantise / LDS-store work with its MFMAs, a piece per MFMA group
 template <int MT, int WN, bool SWIGLU, bool W8>
@@ -113,7 +115,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     constexpr int RB = W8 ? NT / 4 : NT / 8;    // B rows per pass (fp8 rows are 4 chunks of 16 weights)
     constexpr int NB = BN_ROWS / RB;            // 16-byte global B chunks per thread per stage
     constexpr int NBLK = SWIGLU ? 128 : 256;    // output columns per workgroup
-    constexpr int NJ = 8 / WN;                  // 32-wide weight tiles per wave
+    constexpr int NJ = 8 / WN;                  // 32-row units of the weight tile per wave
     static_assert(NA >= 1 && NB >= 2, "tile/thread mismatch");
     // two separate arrays: stores into one stage and reads from the other provably do not alias,
     // which lets the scheduler move them past each other
@@ -276,45 +278,60 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
         }
     };
 
-    // ---- MFMA operand coordinates ----
-    // fragment row = base + lane%32 (bases are multiples of 32); logical chunk = 2*s + lane/32
-    const int frow = lane & 31, fhalf = lane >> 5, fkey = swz(frow);
-    uint32_t tok_off[MT], w_off[NJ];
+    // ---- MFMA operand coordinates (v_mfma_f32_16x16x32_bf16) ----
+    // fragment row = base + lane%16 (bases are multiples of 16); logical chunk = 4*s + lane/16 for
+    // the 32-wide k-step s of the stage: lane l supplies k = 8*(l/16) .. +7 of row l%16
+    const int frow = lane & 15, fquad = lane >> 4, fkey = swz(frow);
+    // The LDS serves a 16-byte read 8 + 8 lanes at a time (lanes 8i.. together with 32+8i..):
+    // such a pair of lane groups must read neighbouring chunks of the same rows, which is what the
+    // swizzle keeps conflict-free, so lane group q takes chunk 0,2,1,3 of the k-step instead of q
+    // (with q the counter SQ_LDS_BANK_CONFLICT reads 22 % of the busy cycles, with this order
+    // 0.3 %).  Both operands use the same order, and a dot product does not care in which order
+    // k is walked.
+    const int fchunk = ((fquad & 1) << 1) | (fquad >> 1);
+    constexpr int TM = 2 * MT, TN = 2 * NJ;       // 16-row token tiles / 16-row weight tiles per wave
+    uint32_t tok_off[TM], w_off[TN];
 #pragma unroll
-    for (int mi = 0; mi < MT; ++mi) tok_off[mi] = (uint32_t)((wm * 32 * MT + 32 * mi + frow) * ROW_B);
+    for (int mi = 0; mi < TM; ++mi) tok_off[mi] = (uint32_t)((wm * 32 * MT + 16 * mi + frow) * ROW_B);
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-        int r = SWIGLU ? ((j < NJ / 2 ? 0 : 128) + wn * (16 * NJ) + 32 * (j % (NJ / 2))) : (wn * (32 * NJ) + 32 * j);
+    for (int j = 0; j < TN; ++j) {
+        int r = SWIGLU ? ((j < TN / 2 ? 0 : 128) + wn * (8 * TN) + 16 * (j % (TN / 2))) : (wn * (16 * TN) + 16 * j);
         w_off[j] = (uint32_t)((r + frow) * ROW_B);
     }
 
-    f32x16 acc[MT][NJ];
+    f32x4 acc[TM][TN];
 #pragma unroll
-    for (int mi = 0; mi < MT; ++mi)
+    for (int mi = 0; mi < TM; ++mi)
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) acc[mi][j] = f32x16{0};
+        for (int j = 0; j < TN; ++j) acc[mi][j] = f32x4{0};
 
-    // Operand fragments are double-buffered in registers: the 16-byte LDS reads of k-step s+1 are
-    // issued before the MFMAs of k-step s.  The pipeline is rotated across the workgroup barrier:
-    // the MFMAs of the LAST k-step of a tile (whose fragments are already in registers) are issued
-    // after the barrier, behind the first LDS reads of the next tile, so the matrix core has work
-    // while those reads are in flight.
-    bf16x8 tf[2][MT], wf[2][NJ];
-    constexpr int NS = BK / 16, LAST = NS - 1;
-    auto read_frags = [&](const uint8_t* As, int s) {
+    // A stage is multiplied in NU sub-phases: k-step s (32 wide) x token part q (TQ tiles), each
+    // TQ x TN MFMAs.  Weight fragments are double-buffered by k-step; token parts ping-pong between
+    // two small buffers.  Slot v of an iteration issues the MFMAs of sub-phase v-2 (the last two
+    // sub-phases of a stage run in the first two slots of the next iteration, across the workgroup
+    // barrier) and then requests the fragments of sub-phase v, whose buffer those MFMAs just freed.
+    constexpr int TQ = (MT >= 2) ? MT / 2 : 1;    // token tiles per part
+    constexpr int NP = TM / TQ;                   // parts per k-step
+    constexpr int NU = 2 * NP;                    // sub-phases per stage
+    bf16x8 wfr[2][TN], tq[2][TQ];
+    auto read_w1 = [&](const uint8_t* As, int s, int j) {
         const uint8_t* Bs = As + A_STAGE;
-        const uint32_t coff = (uint32_t)(((2 * s + fhalf) ^ fkey) << 4);
-#pragma unroll
-        for (int mi = 0; mi < MT; ++mi) tf[s & 1][mi] = *reinterpret_cast<const bf16x8*>(As + tok_off[mi] + coff);
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) wf[s & 1][j] = *reinterpret_cast<const bf16x8*>(Bs + w_off[j] + coff);
+        const uint32_t coff = (uint32_t)(((4 * s + fchunk) ^ fkey) << 4);
+        wfr[s][j] = *reinterpret_cast<const bf16x8*>(Bs + w_off[j] + coff);
     };
-    auto mfmas = [&](int s) {
+    auto read_tq = [&](const uint8_t* As, int u) {
+        const int s = u / NP, q = u % NP;
+        const uint32_t coff = (uint32_t)(((4 * s + fchunk) ^ fkey) << 4);
 #pragma unroll
-        for (int mi = 0; mi < MT; ++mi)
+        for (int i = 0; i < TQ; ++i) tq[u & 1][i] = *reinterpret_cast<const bf16x8*>(As + tok_off[q * TQ + i] + coff);
+    };
+    auto mfma_sub = [&](int u) {
+        const int s = u / NP, q = u % NP;
 #pragma unroll
-            for (int j = 0; j < NJ; ++j)
-                acc[mi][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[s & 1][j], tf[s & 1][mi], acc[mi][j], 0, 0, 0);
+        for (int i = 0; i < TQ; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[q * TQ + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wfr[s][j], tq[u & 1][i], acc[q * TQ + i][j], 0, 0, 0);
     };
     // ---- main loop ----
     // On entry to iteration kt: LDS stage kt&1 holds tile kt and the registers hold tiles kt+1 ..
@@ -369,44 +386,32 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
             rb[set][b] = gload16(m + ((size_t)b_n[b] * K + kofs) * EB + bcol_b);
         }
     };
-    constexpr int MPS = MT * NJ;                  // MFMAs per k-step
-    constexpr int GPS = MPS >= 8 ? 2 : 1;         // MFMA groups per k-step
-    constexpr int MPG = MPS / GPS, NG = NS * GPS; // MFMAs per group, groups per iteration
-    auto mfma_group = [&](int s, int gg) {
-#pragma unroll
-        for (int m = gg * MPG; m < (gg + 1) * MPG; ++m) {
-            const int mi = m / NJ, j = m % NJ;
-            acc[mi][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[s & 1][j], tf[s & 1][mi], acc[mi][j], 0, 0, 0);
-        }
-    };
-    // iteration kt multiplies tile kt out of stage kt&1 (the MFMAs of its k-step t are issued one
-    // step late, behind the fragment reads of step t+1; those of its last step behind the first
-    // reads of the next tile, across the barrier) while tile kt+1 moves from register set kt % PF
-    // (a literal at every call site) into the other stage.
+    constexpr int NG = NU;                        // one group of MFMAs per slot
+    constexpr int WPS = TN / NP;                  // weight fragments of the second k-step read per slot
     auto iteration = [&](int kt, int set, int par) {   // par == kt & 1
         const uint8_t* rd = par ? smem1 : smem0;
         uint8_t* wr = par ? smem0 : smem1;
 #pragma unroll
-        for (int t = 0; t < NS; ++t) {
-            read_frags(rd, t);
+        for (int v = 0; v < NU; ++v) {
+            // group v takes items [v*NI/NG, (v+1)*NI/NG): in order, so the two halves of an fp8
+            // chunk are stored before its registers are refilled
 #pragma unroll
-            for (int gg = 0; gg < GPS; ++gg) {
-                // group g takes items [g*NI/NG, (g+1)*NI/NG): in order, so the two halves of an fp8
-                // chunk are stored before its registers are refilled
-                const int grp = t * GPS + gg;
-#pragma unroll
-                for (int i0 = grp * NI / NG; i0 < (grp + 1) * NI / NG; ++i0) {
-                    // fp8, 4 + 4 items: token chunks and weight half-chunks alternate, so the
-                    // conversion work is spread evenly over the iteration (headline -3 %)
-                    const int i = (W8 && NA == 4 && NI == 8) ? ((i0 & 1) ? NA + (i0 >> 1) : (i0 >> 1)) : i0;
-                    data_item(i, wr, kt, set);
-                }
-                // fp8: the conversion of an item may be scheduled in between the MFMAs of its group
-                if (!W8) __builtin_amdgcn_sched_barrier(0);
-                if (t > 0) mfma_group(t - 1, gg);
-                else if (kt > 0) mfma_group(LAST, gg);
-                __builtin_amdgcn_sched_barrier(0);
+            for (int i0 = v * NI / NG; i0 < (v + 1) * NI / NG; ++i0) {
+                const int i = (W8 && NA == 4 && NI == 8) ? ((i0 & 1) ? NA + (i0 >> 1) : (i0 >> 1)) : i0;
+                data_item(i, wr, kt, set);
             }
+            if (!W8) __builtin_amdgcn_sched_barrier(0);
+            if (v >= 2) mfma_sub(v - 2);
+            else if (kt > 0) mfma_sub(NU - 2 + v);
+            read_tq(rd, v);
+            if (v == 0) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j) read_w1(rd, 0, j);
+            } else if (v >= 2 && v < 2 + NP) {
+#pragma unroll
+                for (int j = (v - 2) * WPS; j < (v - 1) * WPS; ++j) read_w1(rd, 1, j);
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
         __syncthreads();   // (waits for this wave's LDS reads and writes, then for the other waves)
     };
@@ -424,46 +429,43 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     } else {
         for (int kt = 0; kt < nk; ++kt) iteration(kt, 0, kt & 1);
     }
-    mfmas(LAST);
+    mfma_sub(NU - 2);
+    mfma_sub(NU - 1);
 
     // ---- epilogue ----
-    // acc[mi][j][i]: token row = 32*mi + lane%32 of the wave's M range; output column
-    // = tile column base + 8*(i/4) + 4*(lane/32) + i%4, i.e. a lane holds 4 consecutive columns
-    // (8 bytes) of one row per register quad.  Storing those directly would issue 8-byte writes to
-    // 32 different rows per instruction; instead each wave transposes its outputs through its own
+    // acc[mi][j][i]: token row = 16*mi + lane%16 of the wave's M range; output column
+    // = 16*j + 4*(lane/16) + i of the wave's N range, i.e. a lane holds 4 consecutive columns
+    // (8 bytes) of one row per accumulator.  Storing those directly would issue 8-byte writes to
+    // 16 different rows per instruction; instead each wave transposes its outputs through its own
     // slice of the (now idle) LDS stages and writes 16 bytes per lane, whole 64/128-byte row
     // segments per 4/8 lanes.  (All waves passed the loop's last barrier, so no one reads the stages.)
-    constexpr int CW = SWIGLU ? 16 * NJ : 32 * NJ;   // output columns of this wave
+    constexpr int CW = SWIGLU ? 8 * TN : 16 * TN;    // output columns of this wave
     constexpr int RBW = CW * 2;                      // bytes per output row of this wave
     constexpr int CPR = RBW / 16;                    // 16-byte chunks per row (4 or 8)
     constexpr int KSH = CPR == 8 ? 0 : 1;            // swizzle key = (row >> KSH) & (CPR-1)
     uint8_t* ep = ((wave < 4) ? smem0 : smem1) + (wave & 3) * (32 * MT * RBW);
 #pragma unroll
-    for (int mi = 0; mi < MT; ++mi) {
-        const int r = 32 * mi + frow;
-        uint8_t* erow = ep + r * RBW + fhalf * 8;
+    for (int mi = 0; mi < TM; ++mi) {
+        const int r = 16 * mi + frow;
+        uint8_t* erow = ep + r * RBW + (fquad & 1) * 8;
         const int key = (r >> KSH) & (CPR - 1);
 #pragma unroll
-        for (int jj = 0; jj < (SWIGLU ? NJ / 2 : NJ); ++jj) {
+        for (int jj = 0; jj < (SWIGLU ? TN / 2 : TN); ++jj) {
+            u32x2 pk;
+            if (SWIGLU) {
+                float o[4];
 #pragma unroll
-            for (int qd = 0; qd < 4; ++qd) {
-                u32x2 pk;
-                if (SWIGLU) {
-                    float o[4];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        float gv = bf16r(acc[mi][jj][4 * qd + i]);
-                        float uv = bf16r(acc[mi][jj + NJ / 2][4 * qd + i]);
-                        float sg = bf16r(gv * __builtin_amdgcn_rcpf(1.0f + __expf(-gv)));
-                        o[i] = sg * uv;
-                    }
-                    pk = u32x2{pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3])};
-                } else {
-                    pk = u32x2{pack_bf16(acc[mi][jj][4 * qd], acc[mi][jj][4 * qd + 1]),
-                               pack_bf16(acc[mi][jj][4 * qd + 2], acc[mi][jj][4 * qd + 3])};
+                for (int i = 0; i < 4; ++i) {
+                    float gv = bf16r(acc[mi][jj][i]);
+                    float uv = bf16r(acc[mi][jj + TN / 2][i]);
+                    float sg = bf16r(gv * __builtin_amdgcn_rcpf(1.0f + __expf(-gv)));
+                    o[i] = sg * uv;
                 }
-                *reinterpret_cast<u32x2*>(erow + (((4 * jj + qd) ^ key) << 4)) = pk;
+                pk = u32x2{pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3])};
+            } else {
+                pk = u32x2{pack_bf16(acc[mi][jj][0], acc[mi][jj][1]), pack_bf16(acc[mi][jj][2], acc[mi][jj][3])};
             }
+            *reinterpret_cast<u32x2*>(erow + (((2 * jj + (fquad >> 1)) ^ key) << 4)) = pk;
         }
     }
     const int rows_here = min(BM, row_end - row0) - wm * 32 * MT;   // valid rows of this wave
