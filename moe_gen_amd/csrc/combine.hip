@@ -20,7 +20,10 @@ namespace {
 
 constexpr int MAX_K = 16;
 
-template <int MODE>
+// KB: source rows whose 16-byte chunks a lane requests back to back before it starts adding (the
+// sum itself stays in slot order).  The kernel is bound by HBM latency x bytes in flight, and one
+// outstanding load per lane is too few.
+template <int MODE, int KB>
 __global__ __launch_bounds__(256) void combine_kernel(const u32x4* __restrict__ y, const int32_t* __restrict__ pos,
                                                       const int32_t* __restrict__ topk_idx,
                                                       const float* __restrict__ topk_w, const u32x4* __restrict__ shared,
@@ -45,9 +48,18 @@ __global__ __launch_bounds__(256) void combine_kernel(const u32x4* __restrict__ 
     __syncthreads();
     for (int c = threadIdx.x; c < chunks; c += 256) {
         float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-        for (int a = 0; a < k; ++a) {
-            u32x4 v = y[(size_t)s_row[a] * chunks + c];
-            const float w = s_w[a];
+        u32x4 sh = {0, 0, 0, 0}, res = {0, 0, 0, 0};
+        if (shared) sh = shared[(size_t)t * chunks + c];
+        if (residual) res = residual[(size_t)t * chunks + c];   // may alias out: read before this thread writes
+        for (int a0 = 0; a0 < k; a0 += KB) {
+        u32x4 vb[KB];
+#pragma unroll
+        for (int b = 0; b < KB; ++b) vb[b] = y[(size_t)s_row[min(a0 + b, k - 1)] * chunks + c];   // past k: the last row again
+#pragma unroll
+        for (int b = 0; b < KB; ++b) {
+            if (a0 + b >= k) break;
+            const u32x4 v = vb[b];
+            const float w = s_w[a0 + b];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 float lo = __uint_as_float(v[i] << 16), hi = __uint_as_float(v[i] & 0xffff0000u);
@@ -64,8 +76,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const u32x4* __restrict__ 
                 }
             }
         }
-        u32x4 sh = {0, 0, 0, 0};
-        if (shared) sh = shared[(size_t)t * chunks + c];
+        }
         u32x4 o;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -76,8 +87,8 @@ __global__ __launch_bounds__(256) void combine_kernel(const u32x4* __restrict__ 
             }
             o[i] = lo | (hi << 16);
         }
-        if (residual) {  // may alias out: this thread reads its 16 bytes before it writes them
-            const u32x4 r = residual[(size_t)t * chunks + c];
+        if (residual) {
+            const u32x4 r = res;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const uint32_t lo = f32_to_bf16_bits(__uint_as_float(r[i] << 16) + __uint_as_float(o[i] << 16));
@@ -112,12 +123,19 @@ int combine_impl(const void* y, const int32_t* pos, const int32_t* topk_idx, con
     const u32x4* rv = static_cast<const u32x4*>(residual);
     u32x4* ov = static_cast<u32x4*>(out);
     const int chunks = hidden / 8;
-    if (mode == MOE_COMBINE_F32)
-        hipLaunchKernelGGL(combine_kernel<MOE_COMBINE_F32>, grid, block, 0, st, yv, pos, topk_idx, topk_w, sv, rv, top_k, chunks, ov);
-    else if (mode == MOE_COMBINE_BF16_PROD)
-        hipLaunchKernelGGL(combine_kernel<MOE_COMBINE_BF16_PROD>, grid, block, 0, st, yv, pos, topk_idx, topk_w, sv, rv, top_k, chunks, ov);
-    else
-        hipLaunchKernelGGL(combine_kernel<MOE_COMBINE_BF16_SEQ>, grid, block, 0, st, yv, pos, topk_idx, topk_w, sv, rv, top_k, chunks, ov);
+#define MOE_LAUNCH_COMBINE(M, B) \
+    hipLaunchKernelGGL((combine_kernel<M, B>), grid, block, 0, st, yv, pos, topk_idx, topk_w, sv, rv, top_k, chunks, ov)
+#define MOE_LAUNCH_COMBINE_K(M)                          \
+    do {                                                 \
+        if (top_k <= 2) MOE_LAUNCH_COMBINE(M, 2);        \
+        else if (top_k <= 4) MOE_LAUNCH_COMBINE(M, 4);   \
+        else MOE_LAUNCH_COMBINE(M, 8);                   \
+    } while (0)
+    if (mode == MOE_COMBINE_F32) MOE_LAUNCH_COMBINE_K(MOE_COMBINE_F32);
+    else if (mode == MOE_COMBINE_BF16_PROD) MOE_LAUNCH_COMBINE_K(MOE_COMBINE_BF16_PROD);
+    else MOE_LAUNCH_COMBINE_K(MOE_COMBINE_BF16_SEQ);
+#undef MOE_LAUNCH_COMBINE_K
+#undef MOE_LAUNCH_COMBINE
     MOE_HIP_CHECK(hipGetLastError());
     return MOE_OK;
 }
