@@ -88,6 +88,20 @@ def test_grouped_swiglu_vs_oracle(fp8, E, h, I, counts):
     assert er <= TOL
 
 
+@pytest.mark.parametrize("E,h,I,counts", [
+    (1, 192, 320, [300]),            # 256-row tile
+    (2, 192, 320, [100, 30]),        # 128-row tile
+    (4, 320, 192, [5, 9, 0, 20]),    # 64-row tile
+    (1, 64, 64, [70]),               # a single k-stage
+])
+def test_grouped_odd_stage_counts(E, h, I, counts):
+    """bf16 sizes whose K is an odd multiple of 64: the k loop is unrolled by two and ends in a
+    single-stage tail (fp8 sizes are multiples of 128 and never do)."""
+    print(f"grouped odd stages E={E} h={h} I={I} counts={counts}", flush=True)
+    y, ref32, _ = run_case(E, h, I, counts, False, seed=29)
+    assert np.isfinite(y).all() and rel_max(y, ref32) <= TOL
+
+
 @pytest.mark.parametrize("fp8", [False, True])
 @pytest.mark.parametrize("E,mean", [(700, 3), (1024, 2), (600, 200)])
 def test_grouped_many_experts(fp8, E, mean):
