@@ -123,16 +123,22 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     __shared__ __attribute__((aligned(16))) uint8_t smem1[A_STAGE + B_STAGE];
     __shared__ int s_pref[MAX_E + 1];
     __shared__ int s_wtot[NT / 64];
+    __shared__ int s_sel[5];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave & 1, wn = (wave >> 1) % WN;
 
     // ---- M-tile prefix over experts (exclusive scan of ceil(count/BM)) ----
     int run = 0;
+    int my_start = 0, my_mt = 0, my_o0 = 0, my_o1 = 0;   // this thread's expert (of the last pass)
     for (int e0 = 0; e0 < g.E; e0 += NT) {
         int e = e0 + tid;
         int mt = 0;
-        if (e < g.E) mt = (g.offsets[e + 1] - g.offsets[e] + BM - 1) / BM;
+        if (e < g.E) {
+            my_o0 = g.offsets[e];
+            my_o1 = g.offsets[e + 1];
+            mt = (my_o1 - my_o0 + BM - 1) / BM;
+        }
         int inc = mt;
 #pragma unroll
         for (int d = 1; d < 64; d <<= 1) {
@@ -147,12 +153,12 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
             if (w < wave) pre += s_wtot[w];
             tot += s_wtot[w];
         }
-        if (e < g.E) s_pref[e] = pre + inc - mt;
+        my_start = pre + inc - mt;
+        my_mt = mt;
+        if (e < g.E) s_pref[e] = my_start;
         run += tot;
-        __syncthreads();
+        if (g.E > NT) __syncthreads();   // s_wtot is rewritten by the next pass
     }
-    if (tid == 0) s_pref[g.E] = run;
-    __syncthreads();
     const int total = run * g.n_tiles_n;
 
     // ---- XCD-aware id: XCD x (= blockIdx % 8) owns tiles [x*per, (x+1)*per) ----
@@ -161,14 +167,31 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     const int v = (blockIdx.x & 7) * per + slot;
     if (slot >= per || v >= total) return;
     const int q = v / g.n_tiles_n;  // global M-tile number
-    int lo = 0, hi = g.E;           // find e with s_pref[e] <= q < s_pref[e+1]
-    while (hi - lo > 1) {
-        int mid = (lo + hi) >> 1;
-        if (s_pref[mid] <= q) lo = mid; else hi = mid;
+    // find e with prefix[e] <= q < prefix[e+1].  Up to NT experts every thread still holds its own
+    // expert's prefix, tile count and row range: the one that owns q publishes them (one barrier,
+    // no search, no second trip to memory for the offsets).  More experts: binary search in LDS.
+    if (g.E <= NT) {
+        if (tid < g.E && my_start <= q && q < my_start + my_mt) {
+            s_sel[0] = tid; s_sel[1] = my_start; s_sel[2] = my_mt; s_sel[3] = my_o0; s_sel[4] = my_o1;
+        }
+        __syncthreads();
+    } else {
+        if (tid == 0) s_pref[g.E] = run;
+        __syncthreads();
+        int lo = 0, hi = g.E;
+        while (hi - lo > 1) {
+            int mid = (lo + hi) >> 1;
+            if (s_pref[mid] <= q) lo = mid; else hi = mid;
+        }
+        if (tid == 0) {
+            s_sel[0] = lo; s_sel[1] = s_pref[lo]; s_sel[2] = s_pref[lo + 1] - s_pref[lo];
+            s_sel[3] = g.offsets[lo]; s_sel[4] = g.offsets[lo + 1];
+        }
+        __syncthreads();
     }
-    const int e = uni(lo);
-    const int pe = uni(s_pref[e]);
-    const int mt_e = uni(s_pref[e + 1]) - pe;
+    const int e = uni(s_sel[0]);
+    const int pe = uni(s_sel[1]);
+    const int mt_e = uni(s_sel[2]);
     // Inside an expert, tiles are visited in groups of about GM consecutive M tiles (the expert's
     // M tiles split as evenly as possible); within a group the M tile varies fastest.  The ~32
     // workgroups an XCD runs at once then cover ~GM M tiles x 32/GM N tiles and share those
@@ -189,8 +212,8 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
         rem = l2 - gi * sz; gm = base; m0 = extra * (base + 1) + gi * base;
     }
     const int n_tile = rem / gm, m_tile = m0 + (rem - n_tile * gm);
-    const int row0 = uni(g.offsets[e]) + m_tile * BM;
-    const int row_end = uni(g.offsets[e + 1]);
+    const int row0 = uni(s_sel[3]) + m_tile * BM;
+    const int row_end = uni(s_sel[4]);
     const int n0 = n_tile * NBLK;
     const int K = g.K, N = g.N;
 
@@ -483,6 +506,435 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     }
 }
 
+// lane id produced where it is used: the compiler cannot hoist it (and everything derived from it)
+// out of the tile loop and keep it in registers through the k loop
+__device__ __forceinline__ int fresh_lane() {
+    int l;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+    return l;
+}
+
+// Persistent variant of the BM = 256 kernel: one workgroup per CU walks tiles c, c + C, c + 2C, ...
+// of its XCD's range, and the software pipeline runs on across the tile boundary: the last two
+// k-iterations of a tile already fetch the next tile's first two k-stages, the epilogue goes
+// through a small scratch of its own instead of the stages, and the next tile starts with its
+// first stage in LDS and its second in flight.  What a fresh workgroup pays per tile -- launch,
+// tile-prefix scan, pointer chase, first fetch, store drain: 6-8 us against 57 us of k loop for
+// K = 2048 -- is paid once per workgroup, or overlaps the previous tile's work.
+template <bool SWIGLU, bool W8>
+__global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g) {
+    static_assert(W8, "instantiated for fp8 weights only: with bf16 weights it measured no faster than the one-tile kernel");
+    constexpr int MT = 4, WN = 4;
+    constexpr int NT = 128 * WN;                // threads
+    constexpr int BM = 64 * MT;                 // rows per workgroup
+    constexpr int A_STAGE = BM * ROW_B;         // bytes
+    constexpr int B_STAGE = BN_ROWS * ROW_B;
+    constexpr int RA = NT / 8;                  // A rows covered by one pass of the workgroup
+    constexpr int NA = BM / RA;                 // 16-byte A chunks per thread per stage
+    constexpr int RB = W8 ? NT / 4 : NT / 8;    // B rows per pass (fp8 rows are 4 chunks of 16 weights)
+    constexpr int NB = BN_ROWS / RB;            // 16-byte global B chunks per thread per stage
+    constexpr int NBLK = SWIGLU ? 128 : 256;    // output columns per workgroup
+    constexpr int NJ = 8 / WN;                  // 32-row units of the weight tile per wave
+    static_assert(NA >= 1 && NB >= 2, "tile/thread mismatch");
+    // two separate arrays: stores into one stage and reads from the other provably do not alias,
+    // which lets the scheduler move them past each other
+    __shared__ __attribute__((aligned(16))) uint8_t smem0[A_STAGE + B_STAGE];
+    __shared__ __attribute__((aligned(16))) uint8_t smem1[A_STAGE + B_STAGE];
+    __shared__ int s_pref[MAX_E + 1];
+    __shared__ int s_wtot[NT / 64];
+    constexpr int PE = 256;                               // experts this kernel keeps tables for
+    __shared__ int s_off[PE + 1];
+    __shared__ unsigned long long s_ptr[4][PE];           // b0, b1, s0, s1 per expert
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wave_s = uni(wave);                         // scalar copy
+    const int wm = wave_s & 1, wn = (wave_s >> 1) % WN;
+
+    // ---- M-tile prefix over experts (exclusive scan of ceil(count/BM)) ----
+    int run = 0;
+    int my_start = 0, my_mt = 0, my_o0 = 0, my_o1 = 0;   // this thread's expert (of the last pass)
+    for (int e0 = 0; e0 < g.E; e0 += NT) {
+        int e = e0 + tid;
+        int mt = 0;
+        if (e < g.E) {
+            my_o0 = g.offsets[e];
+            my_o1 = g.offsets[e + 1];
+            mt = (my_o1 - my_o0 + BM - 1) / BM;
+            s_off[e] = my_o0;
+            if (e == g.E - 1) s_off[g.E] = my_o1;
+            s_ptr[0][e] = (unsigned long long)(uintptr_t)g.b0[e];
+            s_ptr[1][e] = SWIGLU ? (unsigned long long)(uintptr_t)g.b1[e] : 0ull;
+            s_ptr[2][e] = W8 ? (unsigned long long)(uintptr_t)g.s0[e] : 0ull;
+            s_ptr[3][e] = (W8 && SWIGLU) ? (unsigned long long)(uintptr_t)g.s1[e] : 0ull;
+        }
+        int inc = mt;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            int o = __shfl_up(inc, d);
+            if (lane >= d) inc += o;
+        }
+        if (lane == 63) s_wtot[wave] = inc;
+        __syncthreads();
+        int pre = run, tot = 0;
+#pragma unroll
+        for (int w = 0; w < NT / 64; ++w) {
+            if (w < wave) pre += s_wtot[w];
+            tot += s_wtot[w];
+        }
+        my_start = pre + inc - mt;
+        my_mt = mt;
+        if (e < g.E) s_pref[e] = my_start;
+        run += tot;
+        if (g.E > NT) __syncthreads();   // s_wtot is rewritten by the next pass
+    }
+    if (tid == 0) s_pref[g.E] = run;
+    __syncthreads();
+    const int total = run * g.n_tiles_n;
+
+    // ---- XCD-aware ids: XCD x (= blockIdx % 8) owns tiles [x*per, (x+1)*per); this workgroup takes
+    // every `slots`-th of them ----
+    const int per = (total + 7) / 8;
+    const int xcd = blockIdx.x & 7, slots = gridDim.x >> 3;
+    int slot = blockIdx.x >> 3;
+    if (slot >= per || xcd * per + slot >= total) return;
+    const int K = g.K, N = g.N;
+    constexpr int EB = W8 ? 1 : 2;                        // bytes per weight element
+    const int KB = K >> 7;
+    // the tile whose operands the pipeline is currently FETCHING (the next tile during a tile's last
+    // two iterations) ...
+    const uint8_t *a_ptr[NA], *b_ptr[NB];                 // this thread's chunks at k = 0
+    int srow0 = 0, srow1 = 0;
+    gptr_f32 sc0 = nullptr, sc1 = nullptr;
+    // ... and its output coordinates
+    int row0 = 0, row_end = 0, n0 = 0;
+    int cur_e = 0;                                        // expert of the last tile looked up (tiles only move forward)
+    auto setup = [&](int v) {
+    const int t = wave_s * 64 + fresh_lane();
+    const int lrow = t >> 3, lchunk = t & 7;              // bf16 tiles: row t/8 (+RA i), chunk t%8
+    const int brow = W8 ? (t >> 2) : (t >> 3);            // fp8 tiles: row t/4 (+RB i), 16-byte chunk t%4
+    const int bcol_b = W8 ? ((t & 3) << 4) : ((t & 7) << 4);   // byte offset inside the 64-element k slab
+    const int q = v / g.n_tiles_n;  // global M-tile number
+    while (uni(s_pref[cur_e + 1]) <= q) ++cur_e;        // s_pref[E] = total M tiles > q ends the walk
+    const int e = cur_e;
+    const int pe = uni(s_pref[e]);
+    const int mt_e = uni(s_pref[e + 1]) - pe;
+    // Inside an expert, tiles are visited in groups of about GM consecutive M tiles (the expert's
+    // M tiles split as evenly as possible); within a group the M tile varies fastest.  The ~32
+    // workgroups an XCD runs at once then cover ~GM M tiles x 32/GM N tiles and share those
+    // panels through the XCD's L2: an A panel is fetched once per 32/GM N tiles and a B panel
+    // once per group.  GM = 4 (4 x 8 tiles) balances the two re-fetch factors; measured on 64
+    // experts x 2048 rows (7168 -> 2048, fp8) it fetches 7.0 GiB against 8.75 GiB for GM = 8 or 16.
+    constexpr int GM = 4;
+    const int local = v - pe * g.n_tiles_n;
+    const int ng = max(1, (mt_e + GM / 2) / GM);
+    const int base = mt_e / ng, extra = mt_e - base * ng;      // `extra` groups hold base+1 tiles
+    const int big = (base + 1) * g.n_tiles_n, cut = extra * big;
+    int gm, m0, rem;
+    if (local < cut) {
+        const int gi = local / big;
+        rem = local - gi * big; gm = base + 1; m0 = gi * (base + 1);
+    } else {
+        const int l2 = local - cut, sz = base * g.n_tiles_n, gi = l2 / sz;
+        rem = l2 - gi * sz; gm = base; m0 = extra * (base + 1) + gi * base;
+    }
+    const int n_tile = rem / gm, m_tile = m0 + (rem - n_tile * gm);
+    row0 = uni(s_off[e]) + m_tile * BM;
+    row_end = uni(s_off[e + 1]);
+    n0 = n_tile * NBLK;
+    // ---- per-thread load coordinates ----
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+        int r = min(row0 + lrow + RA * i, row_end - 1);
+        const int src = g.row_map ? ((gptr_i32)(uintptr_t)g.row_map)[r] : r;
+        a_ptr[i] = reinterpret_cast<const uint8_t*>(g.a + (size_t)src * K + lchunk * 8);
+    }
+    const uint8_t* bmat0 = uni_ptr(reinterpret_cast<const void*>((uintptr_t)s_ptr[0][e]));
+    const uint8_t* bmat1 = SWIGLU ? uni_ptr(reinterpret_cast<const void*>((uintptr_t)s_ptr[1][e])) : bmat0;
+    if (W8) {
+        sc0 = (gptr_f32)(uintptr_t)uni_ptr(reinterpret_cast<const void*>((uintptr_t)s_ptr[2][e]));
+        sc1 = SWIGLU ? (gptr_f32)(uintptr_t)uni_ptr(reinterpret_cast<const void*>((uintptr_t)s_ptr[3][e])) : sc0;
+    }
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+        int r = brow + RB * i;                            // row inside the 256-row B tile
+        int n = SWIGLU ? (n0 + (r & 127)) : (n0 + r);
+        const uint8_t* m = (SWIGLU && i >= NB / 2) ? bmat1 : bmat0;  // rows >= 128 of the B tile are the up matrix
+        b_ptr[i] = m + (size_t)min(n, N - 1) * K * EB + bcol_b;
+    }
+    if (W8) {   // block-scale rows: first / second 128 rows of the B tile
+        if (SWIGLU) { srow0 = (n0 >> 7) * KB; srow1 = srow0; }
+        else        { srow0 = (n0 >> 7) * KB; srow1 = min((n0 >> 7) + 1, (N >> 7) - 1) * KB; }
+    }
+    };   // setup
+    const int lrow = tid >> 3, lchunk = tid & 7;
+    const int brow = W8 ? (tid >> 2) : (tid >> 3);
+    const uint32_t a_lds = (uint32_t)(lrow * ROW_B + ((lchunk ^ swz(lrow)) << 4));
+    uint32_t b_lds[2];
+    // fp8: a thread owns chunks 2q and 2q+1 of its row; rows with bit 1 set store them in the
+    // opposite order so that the 16 lanes of one store instruction (4 rows x 4 chunks) spread
+    // over all banks
+    const bool b_swap = W8 && ((brow >> 1) & 1);
+    if (W8) {
+        int qd = tid & 3, sw = swz(brow), first = b_swap ? 1 : 0;
+        b_lds[0] = (uint32_t)(brow * ROW_B + (((2 * qd + first) ^ sw) << 4));
+        b_lds[1] = (uint32_t)(brow * ROW_B + (((2 * qd + 1 - first) ^ sw) << 4));
+    } else {
+        b_lds[0] = (uint32_t)(brow * ROW_B + (((tid & 7) ^ swz(brow)) << 4));
+        b_lds[1] = 0;
+    }
+
+    // PF register sets: global loads run PF tiles ahead of the LDS stores.  One set when the
+    // workgroup is compute bound (BM = 256, which has no registers to spare); two for the smaller
+    // tiles, which mostly stream weights (decode) and where bytes in flight per CU are what
+    // limits the HBM rate.
+    constexpr int PF = (MT <= 2) ? 2 : 1;
+    u32x4 ra[PF][NA], rb[PF][NB];
+    float rs[PF][2];
+    auto gload = [&](int kt, int set) {
+        const size_t kofs = (size_t)kt * BK;
+#pragma unroll
+        for (int i = 0; i < NA; ++i) ra[set][i] = gload16(a_ptr[i] + kofs * 2);
+#pragma unroll
+        for (int i = 0; i < NB; ++i) rb[set][i] = gload16(b_ptr[i] + kofs * EB);
+        if (W8) {
+            rs[set][0] = sc0[srow0 + (kt >> 1)];
+            rs[set][1] = sc1[srow1 + (kt >> 1)];
+        }
+    };
+    auto lds_store = [&](uint8_t* As, int set) {
+        uint8_t* Bs = As + A_STAGE;
+#pragma unroll
+        for (int i = 0; i < NA; ++i) *reinterpret_cast<u32x4*>(As + a_lds + i * RA * ROW_B) = ra[set][i];
+        if (W8) {
+#pragma unroll
+            for (int i = 0; i < NB; ++i) {
+                u32x4 l, h;
+                dequant16(rb[set][i], rs[set][i / (NB / 2)], l, h);
+                *reinterpret_cast<u32x4*>(Bs + b_lds[0] + i * RB * ROW_B) = b_swap ? h : l;
+                *reinterpret_cast<u32x4*>(Bs + b_lds[1] + i * RB * ROW_B) = b_swap ? l : h;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NB; ++i) *reinterpret_cast<u32x4*>(Bs + b_lds[0] + i * RB * ROW_B) = rb[set][i];
+        }
+    };
+
+    // ---- MFMA operand coordinates (v_mfma_f32_16x16x32_bf16) ----
+    // fragment row = base + lane%16 (bases are multiples of 16); logical chunk = 4*s + lane/16 for
+    // the 32-wide k-step s of the stage: lane l supplies k = 8*(l/16) .. +7 of row l%16
+    const int frow = lane & 15, fquad = lane >> 4, fkey = swz(frow);
+    // The LDS serves a 16-byte read 8 + 8 lanes at a time (lanes 8i.. together with 32+8i..):
+    // such a pair of lane groups must read neighbouring chunks of the same rows, which is what the
+    // swizzle keeps conflict-free, so lane group q takes chunk 0,2,1,3 of the k-step instead of q
+    // (with q the counter SQ_LDS_BANK_CONFLICT reads 22 % of the busy cycles, with this order
+    // 0.3 %).  Both operands use the same order, and a dot product does not care in which order
+    // k is walked.
+    const int fchunk = ((fquad & 1) << 1) | (fquad >> 1);
+    constexpr int TM = 2 * MT, TN = 2 * NJ;       // 16-row token tiles / 16-row weight tiles per wave
+    uint32_t tok_off[TM], w_off[TN];
+#pragma unroll
+    for (int mi = 0; mi < TM; ++mi) tok_off[mi] = (uint32_t)((wm * 32 * MT + 16 * mi + frow) * ROW_B);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        int r = SWIGLU ? ((j < TN / 2 ? 0 : 128) + wn * (8 * TN) + 16 * (j % (TN / 2))) : (wn * (16 * TN) + 16 * j);
+        w_off[j] = (uint32_t)((r + frow) * ROW_B);
+    }
+
+    f32x4 acc[TM][TN];
+#pragma unroll
+    for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[mi][j] = f32x4{0};
+
+    // A stage is multiplied in NU sub-phases: k-step s (32 wide) x token part q (TQ tiles), each
+    // TQ x TN MFMAs.  Weight fragments are double-buffered by k-step; token parts ping-pong between
+    // two small buffers.  Slot v of an iteration issues the MFMAs of sub-phase v-2 (the last two
+    // sub-phases of a stage run in the first two slots of the next iteration, across the workgroup
+    // barrier) and then requests the fragments of sub-phase v, whose buffer those MFMAs just freed.
+    constexpr int TQ = (MT >= 2) ? MT / 2 : 1;    // token tiles per part
+    constexpr int NP = TM / TQ;                   // parts per k-step
+    constexpr int NU = 2 * NP;                    // sub-phases per stage
+    bf16x8 wfr[2][TN], tq[2][TQ];
+    auto read_w1 = [&](const uint8_t* As, int s, int j) {
+        const uint8_t* Bs = As + A_STAGE;
+        const uint32_t coff = (uint32_t)(((4 * s + fchunk) ^ fkey) << 4);
+        wfr[s][j] = *reinterpret_cast<const bf16x8*>(Bs + w_off[j] + coff);
+    };
+    auto read_tq = [&](const uint8_t* As, int u) {
+        const int s = u / NP, q = u % NP;
+        const uint32_t coff = (uint32_t)(((4 * s + fchunk) ^ fkey) << 4);
+#pragma unroll
+        for (int i = 0; i < TQ; ++i) tq[u & 1][i] = *reinterpret_cast<const bf16x8*>(As + tok_off[q * TQ + i] + coff);
+    };
+    auto mfma_sub = [&](int u) {
+        const int s = u / NP, q = u % NP;
+#pragma unroll
+        for (int i = 0; i < TQ; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[q * TQ + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wfr[s][j], tq[u & 1][i], acc[q * TQ + i][j], 0, 0, 0);
+    };
+    // ---- main loop ----
+    // On entry to iteration kt: LDS stage kt&1 holds tile kt and the registers hold tiles kt+1 ..
+    // kt+PF (possibly still in flight).  The iteration moves tile kt+1 into the other LDS stage,
+    // refills that register set with tile kt+1+PF and multiplies tile kt.
+    const int nk = K / BK;
+    // One data item = one LDS store's worth of this thread's staged chunks (a 16-byte token chunk,
+    // a 16-byte bf16 weight chunk, or half of a 16-byte fp8 weight chunk -> 8 bf16): store it to the
+    // other stage and, once a chunk's last item is stored, refill its registers with the chunk of
+    // tile kt+1+PF.  The items are spread over the iteration, one per group of MFMAs, so LDS, the
+    // vector-memory pipe and the matrix core see a steady mix instead of bursts; with exact load
+    // waits each item stalls only until its own chunk (requested PF iterations earlier) is there.
+    constexpr int NBI = W8 ? 2 * NB : NB;
+    constexpr int NI = NA + NBI;
+    auto data_item = [&](int i, uint8_t* As, int kn, int set) {   // kn: k-stage (of the tile being fetched) to request
+        uint8_t* Bs = As + A_STAGE;
+        const size_t kofs = (size_t)kn * BK;
+        if (i < NA) {
+            *reinterpret_cast<u32x4*>(As + a_lds + i * RA * ROW_B) = ra[set][i];
+            ra[set][i] = gload16(a_ptr[i] + kofs * 2);
+        } else if (W8) {
+            const int b = (i - NA) >> 1, half = (i - NA) & 1;
+            const float sc = rs[set][b / (NB / 2)];
+            const uint32_t q0 = rb[set][b][2 * half], q1 = rb[set][b][2 * half + 1];
+            const f32x2 c0 = __builtin_amdgcn_cvt_pk_f32_fp8(q0, false), c1 = __builtin_amdgcn_cvt_pk_f32_fp8(q0, true);
+            const f32x2 c2 = __builtin_amdgcn_cvt_pk_f32_fp8(q1, false), c3 = __builtin_amdgcn_cvt_pk_f32_fp8(q1, true);
+            const u32x4 o = {pack_bf16(c0[0] * sc, c0[1] * sc), pack_bf16(c1[0] * sc, c1[1] * sc),
+                             pack_bf16(c2[0] * sc, c2[1] * sc), pack_bf16(c3[0] * sc, c3[1] * sc)};
+            // the first 8 weights go to b_lds[0], the second 8 to b_lds[1]; swapped rows the other way round
+            *reinterpret_cast<u32x4*>(Bs + ((half ^ (b_swap ? 1 : 0)) ? b_lds[1] : b_lds[0]) + b * RB * ROW_B) = o;
+            if (half == 1) {
+                rb[set][b] = gload16(b_ptr[b] + kofs * EB);
+                if (b / (NB / 2) == 0) rs[set][0] = sc0[srow0 + (kn >> 1)];
+                else rs[set][1] = sc1[srow1 + (kn >> 1)];
+            }
+        } else {
+            const int b = i - NA;
+            *reinterpret_cast<u32x4*>(Bs + b_lds[0] + b * RB * ROW_B) = rb[set][b];
+            rb[set][b] = gload16(b_ptr[b] + kofs * EB);
+        }
+    };
+    constexpr int NG = NU;                        // one group of MFMAs per slot
+    constexpr int WPS = TN / NP;                  // weight fragments of the second k-step read per slot
+    auto iteration = [&](int kt, int kn, int set, int par) {   // par == kt & 1
+        const uint8_t* rd = par ? smem1 : smem0;
+        uint8_t* wr = par ? smem0 : smem1;
+#pragma unroll
+        for (int v = 0; v < NU; ++v) {
+            // group v takes items [v*NI/NG, (v+1)*NI/NG): in order, so the two halves of an fp8
+            // chunk are stored before its registers are refilled
+#pragma unroll
+            for (int i0 = v * NI / NG; i0 < (v + 1) * NI / NG; ++i0) {
+                const int i = (W8 && NA == 4 && NI == 8) ? ((i0 & 1) ? NA + (i0 >> 1) : (i0 >> 1)) : i0;
+                data_item(i, wr, kn, set);
+            }
+            if (!W8) __builtin_amdgcn_sched_barrier(0);
+            if (v >= 2) mfma_sub(v - 2);
+            else if (kt > 0) mfma_sub(NU - 2 + v);
+            read_tq(rd, v);
+            if (v == 0) {
+#pragma unroll
+                for (int j = 0; j < TN; ++j) read_w1(rd, 0, j);
+            } else if (v >= 2 && v < 2 + NP) {
+#pragma unroll
+                for (int j = (v - 2) * WPS; j < (v - 1) * WPS; ++j) read_w1(rd, 1, j);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();   // (waits for this wave's LDS reads and writes, then for the other waves)
+    };
+    // ---- tiles ----
+    static_assert(PF == 1, "the tile hand-over below assumes one register set");
+    setup(xcd * per + slot);
+    gload(0, 0);
+    lds_store(smem0, 0);
+    gload(1, 0);
+    __syncthreads();
+    constexpr int CW = SWIGLU ? 8 * TN : 16 * TN;    // output columns of this wave
+    constexpr int RBW = CW * 2;                      // bytes per output row of this wave
+    constexpr int CPR = RBW / 16;                    // 16-byte chunks per row (4 or 8)
+    constexpr int KSH = CPR == 8 ? 0 : 1;            // swizzle key = (row >> KSH) & (CPR-1)
+    constexpr int RPP = 64 / CPR;                    // rows per read-back pass
+    for (;;) {
+        const int out_row0 = row0, out_row_end = row_end, out_n0 = n0;
+#pragma unroll
+        for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[mi][j] = f32x4{0};
+        // k-iterations 0 .. nk-3 fetch this tile's stages 2 .. nk-1 (nk is even and >= 2); the last two
+        // fetch stages 0 and 1 of the next tile, whose coordinates are looked up right before them
+        // (no tile left: this tile's last stage again, stored where nobody reads it); no branch around
+        // the loads.  (With the hand-over folded into the one loop body the kernel needs no spill at
+        // all, but measured 3 % slower on the gate/up shape.)
+        bool more = false;
+        {
+            for (int kt = 0; kt + 2 <= nk - 2; kt += 2) {
+                iteration(kt, kt + 2, 0, 0);
+                iteration(kt + 1, kt + 3, 0, 1);
+            }
+            slot += slots;
+            more = slot < per && xcd * per + slot < total;
+            setup(xcd * per + (more ? slot : slot - slots));
+            iteration(nk - 2, more ? 0 : nk - 1, 0, 0);
+            iteration(nk - 1, more ? 1 : nk - 1, 0, 1);
+        }
+        mfma_sub(NU - 2);
+        mfma_sub(NU - 1);
+
+        // ---- epilogue ----
+        // acc[mi][j][i]: token row = 16*mi + lane%16 of the wave's M range; output column
+        // = 16*j + 4*(lane/16) + i of the wave's N range, i.e. a lane holds 4 consecutive columns
+        // (8 bytes) of one row per accumulator.  Stage 0 already holds the next tile; stage 1 is idle
+        // until the next tile's first iteration writes it, so each wave transposes its outputs through
+        // its 8 KiB slice of stage 1 (64 or 128 rows at a time) and writes 16 bytes per lane, whole
+        // 64/128-byte row segments per 4/8 lanes.
+        const int rows_here = min(BM, out_row_end - out_row0) - wm * 32 * MT;   // valid rows of this wave
+        const int ncol0 = out_n0 + wn * CW;
+        const int el = fresh_lane();
+        const int efrow = el & 15, efquad = el >> 4, rr = el / CPR, cc = el % CPR;
+        uint8_t* ep = smem1 + wave_s * 8192;
+        constexpr int RPW = 8192 / RBW;                  // rows per pass (128 or 64)
+#pragma unroll
+        for (int pass = 0; pass < 32 * MT / RPW; ++pass) {
+#pragma unroll
+            for (int ml = 0; ml < RPW / 16; ++ml) {
+                const int mi = pass * (RPW / 16) + ml;
+                const int r = 16 * ml + efrow;
+                uint8_t* erow = ep + r * RBW + (efquad & 1) * 8;
+                const int key = (r >> KSH) & (CPR - 1);
+#pragma unroll
+                for (int jj = 0; jj < (SWIGLU ? TN / 2 : TN); ++jj) {
+                    u32x2 pk;
+                    if (SWIGLU) {
+                        float o[4];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            float gv = bf16r(acc[mi][jj][i]);
+                            float uv = bf16r(acc[mi][jj + TN / 2][i]);
+                            float sg = bf16r(gv * __builtin_amdgcn_rcpf(1.0f + __expf(-gv)));
+                            o[i] = sg * uv;
+                        }
+                        pk = u32x2{pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3])};
+                    } else {
+                        pk = u32x2{pack_bf16(acc[mi][jj][0], acc[mi][jj][1]), pack_bf16(acc[mi][jj][2], acc[mi][jj][3])};
+                    }
+                    *reinterpret_cast<u32x2*>(erow + (((2 * jj + (efquad >> 1)) ^ key) << 4)) = pk;
+                }
+            }
+#pragma unroll
+            for (int ps = 0; ps < RPW / RPP; ++ps) {
+                const int r = rr + RPP * ps;
+                const u32x4 v = *reinterpret_cast<const u32x4*>(ep + r * RBW + ((cc ^ ((r >> KSH) & (CPR - 1))) << 4));
+                if (pass * RPW + r < rows_here && ncol0 + cc * 8 < N)
+                    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(g.c + (size_t)(out_row0 + wm * 32 * MT + pass * RPW + r) * N + ncol0 + cc * 8));
+            }
+        }
+        if (!more) return;
+        __syncthreads();   // every wave has read its outputs back: the next tile may write stage 1
+    }
+}
+
+
 template <int MT, int WN, bool SWIGLU, bool W8>
 int launch_one(const GemmArgs& g, int n_rows, hipStream_t st) {
     constexpr int BM = 64 * MT;
@@ -498,9 +950,37 @@ int launch_one(const GemmArgs& g, int n_rows, hipStream_t st) {
     return MOE_OK;
 }
 
+// CUs of the current device (the persistent kernel runs one workgroup on each)
+inline int cu_count() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
+template <bool SWIGLU, bool W8>
+int launch_persistent(const GemmArgs& g, int n_rows, hipStream_t st) {
+    const long max_mtiles = (long)n_rows / 256 + g.E;
+    long grid = ((max_mtiles * g.n_tiles_n + 7) / 8) * 8;
+    const long ncu = (cu_count() / 8) * 8;
+    if (grid > ncu) grid = ncu;
+    hipLaunchKernelGGL((grouped_gemm_persistent_kernel<SWIGLU, W8>), dim3((unsigned)grid), dim3(512), 0, st, g);
+    MOE_HIP_CHECK(hipGetLastError());
+    return MOE_OK;
+}
+
 template <bool SWIGLU, bool W8>
 int launch_mt(const GemmArgs& g, int n_rows, hipStream_t st) {
     const long mean = g.E > 0 ? (long)n_rows / g.E : 0;
+    if constexpr (W8) {
+        // fp8 K is a multiple of 128, i.e. an even number of k-stages, which the hand-over needs
+        if (mean >= 192 && g.K % 128 == 0 && g.E <= 256 && cu_count() >= 8) return launch_persistent<SWIGLU, W8>(g, n_rows, st);
+    }
     // The counts themselves live on the device; only their mean is known here.  Routing is
     // uneven, so around a mean of 64 rows some experts exceed 64 and would stream their weights
     // once per 64-row tile: 128-row tiles from a mean of 48 (Mixtral-8x22B decode, 256 tokens:

@@ -128,6 +128,19 @@ def test_grouped_too_many_experts_is_an_error():
 
 
 @pytest.mark.parametrize("fp8", [False, True])
+def test_grouped_more_tiles_than_cus(fp8):
+    """808 gate/up tiles and 404 down tiles of 256 rows on 256 CUs: with fp8 weights every persistent
+    workgroup hands its pipeline over from tile to tile (different experts, a ragged last tile, a
+    10-row expert in between); rows are gathered through a row map."""
+    print(f"grouped more tiles than CUs fp8={fp8}", flush=True)
+    y, ref32, _ = run_case(4, 1024, 1024, [9000, 7000, 10, 9000], fp8, seed=31, use_row_map=True)
+    assert np.isfinite(y).all()
+    err = rel_max(y, ref32)
+    print(f"  max-rel vs fp32 {err:.3e}", flush=True)
+    assert err <= TOL
+
+
+@pytest.mark.parametrize("fp8", [False, True])
 def test_grouped_swiglu_row_map(fp8):
     y, ref32, _ = run_case(4, 256, 256, [100, 0, 300, 77], fp8, seed=23, use_row_map=True)
     assert rel_max(y, ref32) <= TOL
