@@ -192,7 +192,7 @@ def decoder_half_run(w, blk, x, steps: int):
 # (two runs; FETCH_SIZE scaled by 2.0, the factor a plain copy kernel of known size showed on this
 # box, WRITE_SIZE by 1.0).  bench.py cannot run the profiler on itself, so the figures are recorded
 # here from profiles/ for the workloads that were profiled; None elsewhere.
-MEASURED_TRAFFIC_BYTES = {"deepseek_v3_w8a16": 34.7e9}   # profiles/pmc_traffic_deepseek_v3_w8a16_65536.md
+MEASURED_TRAFFIC_BYTES = {"deepseek_v3_w8a16": 23.3e9}   # profiles/pmc_traffic_deepseek_v3_w8a16_65536.md
 
 
 def run_workload(name: str, args, with_cpu: bool):
@@ -253,7 +253,9 @@ def run_workload(name: str, args, with_cpu: bool):
                    "weights": "fp8-e4m3fn + 128x128 fp32 scales, dequantised to bf16 ahead of MFMA" if w.fp8 else "bf16",
                    "gather": "materialized" if args.materialize else "fused into the GEMM A-operand load"},
         "roofline": {"bound": "mfma",
-                     "kernel": f"grouped_gemm_kernel<MT={mt},WN=4,SWIGLU=true,W8={'true' if w.fp8 else 'false'}> (gate/up + SiLU*mul)",
+                     "kernel": ("grouped_gemm_persistent_kernel<SWIGLU=true,W8=true> (gate/up + SiLU*mul)"
+                                if w.fp8 and mt == 4 and w.E <= 256 else
+                                f"grouped_gemm_kernel<MT={mt},WN=4,SWIGLU=true,W8={'true' if w.fp8 else 'false'}> (gate/up + SiLU*mul)"),
                      "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(name),
                      "frac_of_fp8_peak": achieved / PEAK_FP8_TFLOPS,

@@ -926,7 +926,13 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
                 const int r = rr + RPP * ps;
                 const u32x4 v = *reinterpret_cast<const u32x4*>(ep + r * RBW + ((cc ^ ((r >> KSH) & (CPR - 1))) << 4));
                 if (pass * RPW + r < rows_here && ncol0 + cc * 8 < N)
-                    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(g.c + (size_t)(out_row0 + wm * 32 * MT + pass * RPW + r) * N + ncol0 + cc * 8));
+                {
+                    u32x4* dst = reinterpret_cast<u32x4*>(g.c + (size_t)(out_row0 + wm * 32 * MT + pass * RPW + r) * N + ncol0 + cc * 8);
+                    // down projection: whole 128-byte lines per 8 lanes, written non-temporally (the
+                    // pipeline's next load waits also cover these stores; -0.8 %).  The gate/up
+                    // launch writes half lines per wave: plain stores, so that L2 merges the halves.
+                    if (SWIGLU) *dst = v; else __builtin_nontemporal_store(v, dst);
+                }
             }
         }
         if (!more) return;
