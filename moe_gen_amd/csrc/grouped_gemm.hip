@@ -523,7 +523,6 @@ __device__ __forceinline__ int fresh_lane() {
 // K = 2048 -- is paid once per workgroup, or overlaps the previous tile's work.
 template <bool SWIGLU, bool W8>
 __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g) {
-    static_assert(W8, "instantiated for fp8 weights only: with bf16 weights it measured no faster than the one-tile kernel");
     constexpr int MT = 4, WN = 4;
     constexpr int NT = 128 * WN;                // threads
     constexpr int BM = 64 * MT;                 // rows per workgroup
@@ -863,11 +862,12 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
             for (int j = 0; j < TN; ++j) acc[mi][j] = f32x4{0};
         // k-iterations 0 .. nk-3 fetch this tile's stages 2 .. nk-1 (nk is even and >= 2); the last two
         // fetch stages 0 and 1 of the next tile, whose coordinates are looked up right before them
-        // (no tile left: this tile's last stage again, stored where nobody reads it); no branch around
-        // the loads.  (With the hand-over folded into the one loop body the kernel needs no spill at
-        // all, but measured 3 % slower on the gate/up shape.)
+        // (no tile left: this tile's last stage again, stored where nobody reads it).
         bool more = false;
-        {
+        if (W8) {
+            // fp8: the k loop is unrolled by two with literal stage parities, and the two hand-over
+            // iterations are a copy of their own behind it (folded into the loop body the kernel
+            // needs no spill at all, but the gate/up shape measured 3 % slower)
             for (int kt = 0; kt + 2 <= nk - 2; kt += 2) {
                 iteration(kt, kt + 2, 0, 0);
                 iteration(kt + 1, kt + 3, 0, 1);
@@ -877,6 +877,20 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
             setup(xcd * per + (more ? slot : slot - slots));
             iteration(nk - 2, more ? 0 : nk - 1, 0, 0);
             iteration(nk - 1, more ? 1 : nk - 1, 0, 1);
+        } else {
+            // bf16 (4 instead of 2 weight chunks in flight per thread) has no registers for a second
+            // copy of the iteration: one rolled loop, the lookup under a uniform branch in front of
+            // the hand-over iterations (a copy of its own spills 30-46 registers, and every reload is a
+            // vmcnt(0) that drains the prefetch)
+            for (int kt = 0; kt < nk; ++kt) {
+                if (kt == nk - 2) {
+                    slot += slots;
+                    more = slot < per && xcd * per + slot < total;
+                    setup(xcd * per + (more ? slot : slot - slots));
+                }
+                const int kn = kt + 2 < nk ? kt + 2 : (more ? kt + 2 - nk : nk - 1);
+                iteration(kt, kn, 0, kt & 1);
+            }
         }
         mfma_sub(NU - 2);
         mfma_sub(NU - 1);
@@ -983,10 +997,9 @@ int launch_persistent(const GemmArgs& g, int n_rows, hipStream_t st) {
 template <bool SWIGLU, bool W8>
 int launch_mt(const GemmArgs& g, int n_rows, hipStream_t st) {
     const long mean = g.E > 0 ? (long)n_rows / g.E : 0;
-    if constexpr (W8) {
-        // fp8 K is a multiple of 128, i.e. an even number of k-stages, which the hand-over needs
-        if (mean >= 192 && g.K % 128 == 0 && g.E <= 256 && cu_count() >= 8) return launch_persistent<SWIGLU, W8>(g, n_rows, st);
-    }
+    // the persistent kernel needs an even number of k-stages for its hand-over (fp8 sizes always have
+    // one) and keeps per-expert tables for up to 256 experts
+    if (mean >= 192 && g.K % 128 == 0 && g.E <= 256 && cu_count() >= 8) return launch_persistent<SWIGLU, W8>(g, n_rows, st);
     // The counts themselves live on the device; only their mean is known here.  Routing is
     // uneven, so around a mean of 64 rows some experts exceed 64 and would stream their weights
     // once per 64-row tile: 128-row tiles from a mean of 48 (Mixtral-8x22B decode, 256 tokens:
