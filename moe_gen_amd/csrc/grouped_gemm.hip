@@ -19,6 +19,9 @@
 // Workgroup ids are dealt round-robin to the 8 XCDs by the hardware; the id is remapped
 // so that each XCD owns a contiguous range of tiles (same expert, neighbouring M/N
 // tiles), which is what makes its private L2 hold the A and B panels that are re-read.
+// For 256-row tiles (grouped_gemm_persistent_kernel) the launch has one workgroup per CU
+// instead, each walks every 32nd tile of its XCD's range, and the k pipeline runs on from
+// one tile into the next.
 //
 // Workgroup = 8 waves (2 along M, 4 along N), two per SIMD.  Per wave 2*MT x 4 MFMA tiles of
 // 16x16 (v_mfma_f32_16x16x32_bf16), i.e. up to 128x64 outputs and 128 fp32 accumulators.  On
