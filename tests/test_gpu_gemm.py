@@ -77,6 +77,7 @@ def run_case(E, h, I, counts, fp8, seed, use_row_map=False):
     (8, 256, 256, [3, 0, 40, 17, 0, 1, 64, 9]),        # mean < 48 rows per expert: the 64-row tile
     (6, 384, 128, [70, 2, 0, 33, 1, 5]),
     (2, 128, 128, [1, 0]),
+    (4, 384, 256, [300, 500, 0, 260]),                 # 256-row tiles, ragged last N tile of the down projection
 ])
 def test_grouped_swiglu_vs_oracle(fp8, E, h, I, counts):
     print(f"grouped fp8={fp8} E={E} h={h} I={I} counts={counts}", flush=True)
@@ -93,6 +94,7 @@ def test_grouped_swiglu_vs_oracle(fp8, E, h, I, counts):
     (2, 192, 320, [100, 30]),        # 128-row tile
     (4, 320, 192, [5, 9, 0, 20]),    # 64-row tile
     (1, 64, 64, [70]),               # a single k-stage
+    (4, 384, 320, [300, 500, 0, 260]),   # gate/up: even stage count, ragged last N tile; down: 5 stages
 ])
 def test_grouped_odd_stage_counts(E, h, I, counts):
     """bf16 sizes whose K is an odd multiple of 64: the k loop is unrolled by two and ends in a
