@@ -20,8 +20,8 @@
 // so that each XCD owns a contiguous range of tiles (same expert, neighbouring M/N
 // tiles), which is what makes its private L2 hold the A and B panels that are re-read.
 // For 256-row tiles (grouped_gemm_persistent_kernel) the launch has one workgroup per CU
-// instead, each walks every 32nd tile of its XCD's range, and the k pipeline runs on from
-// one tile into the next.
+// instead, groups of 32 consecutive tiles go round-robin to the XCDs, and a workgroup's k
+// pipeline runs on from one of its tiles into the next.
 //
 // Workgroup = 8 waves (2 along M, 4 along N), two per SIMD.  Per wave 2*MT x 4 MFMA tiles of
 // 16x16 (v_mfma_f32_16x16x32_bf16), i.e. up to 128x64 outputs and 128 fp32 accumulators.  On
@@ -517,8 +517,8 @@ __device__ __forceinline__ int fresh_lane() {
     return l;
 }
 
-// Persistent variant of the BM = 256 kernel: one workgroup per CU walks tiles c, c + C, c + 2C, ...
-// of its XCD's range, and the software pipeline runs on across the tile boundary: the last two
+// Persistent variant of the BM = 256 kernel: one workgroup per CU walks its share of the tiles, and
+// the software pipeline runs on across the tile boundary: the last two
 // k-iterations of a tile already fetch the next tile's first two k-stages, the epilogue goes
 // through a small scratch of its own instead of the stages, and the next tile starts with its
 // first stage in LDS and its second in flight.  What a fresh workgroup pays per tile -- launch,
@@ -593,12 +593,17 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
     __syncthreads();
     const int total = run * g.n_tiles_n;
 
-    // ---- XCD-aware ids: XCD x (= blockIdx % 8) owns tiles [x*per, (x+1)*per); this workgroup takes
-    // every `slots`-th of them ----
-    const int per = (total + 7) / 8;
+    // ---- XCD-aware ids.  The `slots` workgroups of an XCD (= blockIdx % 8) work on `slots`
+    // consecutive tiles at a time (4 M tiles x 8 N tiles of one expert, sharing panels through the
+    // XCD's L2), and such groups go round-robin to the XCDs: group G belongs to XCD G % 8, so at any
+    // time the chip works on 8 neighbouring groups -- one or two experts -- whose panels the 256 MiB
+    // memory-side cache then holds for the other XCDs (each XCD on a far-apart range of its own:
+    // headline +2.5 %, Mixtral-8x7B +2.7 % slower).  The workgroup in slot c of its XCD takes tile c
+    // of the XCD's 1st, 2nd, ... group.
     const int xcd = blockIdx.x & 7, slots = gridDim.x >> 3;
     int slot = blockIdx.x >> 3;
-    if (slot >= per || xcd * per + slot >= total) return;
+    auto tile_of = [&](int sl) { return ((sl / slots) * 8 + xcd) * slots + (sl % slots); };
+    if (tile_of(slot) >= total) return;
     const int K = g.K, N = g.N;
     constexpr int EB = W8 ? 1 : 2;                        // bytes per weight element
     const int KB = K >> 7;
@@ -847,7 +852,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
     };
     // ---- tiles ----
     static_assert(PF == 1, "the tile hand-over below assumes one register set");
-    setup(xcd * per + slot);
+    setup(tile_of(slot));
     gload(0, 0);
     lds_store(smem0, 0);
     gload(1, 0);
@@ -876,8 +881,8 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
                 iteration(kt + 1, kt + 3, 0, 1);
             }
             slot += slots;
-            more = slot < per && xcd * per + slot < total;
-            setup(xcd * per + (more ? slot : slot - slots));
+            more = tile_of(slot) < total;
+            setup(tile_of(more ? slot : slot - slots));
             iteration(nk - 2, more ? 0 : nk - 1, 0, 0);
             iteration(nk - 1, more ? 1 : nk - 1, 0, 1);
         } else {
@@ -888,8 +893,8 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
             for (int kt = 0; kt < nk; ++kt) {
                 if (kt == nk - 2) {
                     slot += slots;
-                    more = slot < per && xcd * per + slot < total;
-                    setup(xcd * per + (more ? slot : slot - slots));
+                    more = tile_of(slot) < total;
+                    setup(tile_of(more ? slot : slot - slots));
                 }
                 const int kn = kt + 2 < nk ? kt + 2 : (more ? kt + 2 - nk : nk - 1);
                 iteration(kt, kn, 0, kt & 1);
