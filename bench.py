@@ -254,7 +254,7 @@ def run_workload(name: str, args, with_cpu: bool):
                    "gather": "materialized" if args.materialize else "fused into the GEMM A-operand load"},
         "roofline": {"bound": "mfma",
                      "kernel": (f"grouped_gemm_persistent_kernel<SWIGLU=true,W8={'true' if w.fp8 else 'false'}> (gate/up + SiLU*mul)"
-                                if mt == 4 and w.E <= 256 and w.h % 128 == 0 else
+                                if mt == 4 and w.E <= 512 and w.h % 128 == 0 else
                                 f"grouped_gemm_kernel<MT={mt},WN=4,SWIGLU=true,W8={'true' if w.fp8 else 'false'}> (gate/up + SiLU*mul)"),
                      "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(name),

@@ -544,7 +544,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
     __shared__ __attribute__((aligned(16))) uint8_t smem1[A_STAGE + B_STAGE];
     __shared__ int s_pref[MAX_E + 1];
     __shared__ int s_wtot[NT / 64];
-    constexpr int PE = 256;                               // experts this kernel keeps tables for
+    constexpr int PE = 512;                               // experts this kernel keeps tables for (18 KiB of LDS)
     __shared__ int s_off[PE + 1];
     __shared__ unsigned long long s_ptr[4][PE];           // b0, b1, s0, s1 per expert
 
@@ -1006,8 +1006,8 @@ template <bool SWIGLU, bool W8>
 int launch_mt(const GemmArgs& g, int n_rows, hipStream_t st) {
     const long mean = g.E > 0 ? (long)n_rows / g.E : 0;
     // the persistent kernel needs an even number of k-stages for its hand-over (fp8 sizes always have
-    // one) and keeps per-expert tables for up to 256 experts
-    if (mean >= 192 && g.K % 128 == 0 && g.E <= 256 && cu_count() >= 8) return launch_persistent<SWIGLU, W8>(g, n_rows, st);
+    // one) and keeps per-expert tables for up to 512 experts
+    if (mean >= 192 && g.K % 128 == 0 && g.E <= 512 && cu_count() >= 8) return launch_persistent<SWIGLU, W8>(g, n_rows, st);
     // The counts themselves live on the device; only their mean is known here.  Routing is
     // uneven, so around a mean of 64 rows some experts exceed 64 and would stream their weights
     // once per 64-row tile: 128-row tiles from a mean of 48 (Mixtral-8x22B decode, 256 tokens:

@@ -105,10 +105,11 @@ def test_grouped_odd_stage_counts(E, h, I, counts):
 
 
 @pytest.mark.parametrize("fp8", [False, True])
-@pytest.mark.parametrize("E,mean", [(700, 3), (1024, 2), (600, 200)])
+@pytest.mark.parametrize("E,mean", [(700, 3), (1024, 2), (600, 200), (400, 200)])
 def test_grouped_many_experts(fp8, E, mean):
     """More experts than threads in a workgroup (the M-tile prefix scan takes two passes), up to the
-    maximum of 1024, with empty experts sprinkled in; the last case takes the 256-row tile."""
+    maximum of 1024, with empty experts sprinkled in; the last two cases take the 256-row tile (400
+    experts: the persistent kernel with its per-expert tables in LDS; 600: one workgroup per tile)."""
     print(f"grouped many experts fp8={fp8} E={E} mean={mean}", flush=True)
     rng = np.random.default_rng(E)
     counts = rng.poisson(mean, E)
