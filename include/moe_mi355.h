@@ -122,7 +122,8 @@ int moe_dispatch(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k, int32
  *   offsets   device int32 [E+1] (as written by moe_dispatch); offsets[E] <= n_rows
  *   act       device bf16 [n_rows, I]  scratch for a
  *   y         device bf16 [n_rows, h]  out
- *   workspace device, at least moe_grouped_workspace_bytes(n_rows, E) bytes
+ *   workspace reserved: the kernels find their tiles from offsets[] on the device and need no
+ *             scratch; NULL / 0 is accepted (moe_grouped_workspace_bytes reports the reserve)
  *   phases    MOE_PHASE_GATE_UP (writes act), MOE_PHASE_DOWN (reads act, writes y) or
  *             MOE_PHASE_BOTH; the two launches can be issued (and timed) separately
  * Requires h % 64 == 0 and I % 64 == 0.
