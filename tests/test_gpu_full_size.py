@@ -33,7 +33,8 @@ def subset_reference(blk, w, x2d, tokens, idx, wts):
     return out
 
 
-@pytest.mark.parametrize("name", ["deepseek_v3_w8a16", "deepseek_v2_236b", "mixtral_8x22b"])
+@pytest.mark.parametrize("name", ["deepseek_v3_w8a16", "deepseek_v2_236b", "mixtral_8x22b", "mixtral_8x7b",
+                                  "deepseek_v2_lite", "mixtral_8x22b_decode"])
 def test_full_size_layer(name):
     from moe_gen_amd import synthetic
     w = synthetic.WORKLOADS[name]
