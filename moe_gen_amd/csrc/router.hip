@@ -233,10 +233,13 @@ __device__ void route_token(const float* row, const float* __restrict__ bias, co
 // Two logit engines share the kernel:
 //  SMALL == false: v_mfma_f32_32x32x1_2b_f32.  NEB: 32-expert MFMA blocks per wave (1 or 2);
 //                  WE / WT: waves along experts / tokens.
-//  SMALL == true : v_mfma_f32_4x4x1_16b_f32 for E <= 16 (Mixtral's 8 experts): one instruction is
-//                  64 tokens x 4 experts in 8 cycles, so nothing is padded to 32 experts and the
-//                  sequential-in-k dependency chain is 8x shorter.  NEB = groups of 4 experts (1..4),
-//                  WE = 1.
+//  SMALL == true : v_mfma_f32_4x4x1_16b_f32: one instruction is 64 tokens x 4 experts in 8 cycles, so
+//                  nothing is padded to 32 experts and the sequential-in-k dependency chain is 8x
+//                  shorter.  NEB = groups of 4 experts per wave (1..4), WE waves along experts.  Used
+//                  for E <= 16 (Mixtral's 8 experts) and, with few tokens, up to 64 experts: a handful
+//                  of workgroups cannot hide the 64-cycle latency of the 32x32 chain, and 16 experts
+//                  per wave spread the work over twice as many waves (it reads 8x the LDS operand
+//                  bytes per MAC, which is why many tokens stay on the 32x32 engine).
 // Global loads run two k-stages ahead in registers (two register sets, loop unrolled by two), which
 // is what hides the load latency when only a few workgroups exist (small token counts).
 template <bool SMALL, int NEB, int WE, int WT>
@@ -248,7 +251,7 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     constexpr int LDK = KC + 4;          // padded fp32 row stride: conflict-free 16-byte reads
     constexpr int NT = 64 * WE * WT;  // threads
     constexpr int BT = 64 * WT;       // tokens per block
-    constexpr int EP = SMALL ? 4 * NEB : 32 * NEB * WE;  // padded experts per block
+    constexpr int EP = SMALL ? 4 * NEB * WE : 32 * NEB * WE;  // padded experts per block
     constexpr int XCH = BT * (KC / 8), WCH = EP * (KC / 8);  // 16-byte chunks per stage
     constexpr int XPT = (XCH + NT - 1) / NT, WPT = (WCH + NT - 1) / NT;
     constexpr int TILE_F = (BT + EP) * LDK, LOGIT_F = BT * EP;
@@ -313,7 +316,7 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
 #pragma unroll
     for (int j = 0; j < (SMALL ? NEB : 1); ++j) acc4[j] = f32x4{0, 0, 0, 0};
     const float* a_row = Xs + (wt * 64 + lane) * LDK;
-    const float* b0_row = SMALL ? Ws + (lane & 3) * LDK
+    const float* b0_row = SMALL ? Ws + (we * 4 * NEB + (lane & 3)) * LDK
                                 : Ws + (NEB == 2 ? (we * 64 + lane) : (we * 32 + (lane & 31))) * LDK;
     const float* b1_row = Ws + (we * 64 + (lane ^ 32)) * LDK;  // only read when !SMALL && NEB == 2
 
@@ -378,7 +381,7 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
 #pragma unroll
         for (int j = 0; j < NEB; ++j)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) lg[(wt * 64 + 4 * (lane >> 2) + i) * EP + 4 * j + (lane & 3)] = acc4[j][i];
+            for (int i = 0; i < 4; ++i) lg[(wt * 64 + 4 * (lane >> 2) + i) * EP + we * 4 * NEB + 4 * j + (lane & 3)] = acc4[j][i];
     } else {
         // in block b of the 2-block MFMA result, register 16*b+i of lane l is row
         // 8*(i/4) + 4*(l/32) + i%4, column l%32
@@ -402,7 +405,9 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
 
     // selection, a lane group per token: 16 lanes for E <= 16, 32 for E <= 32, else the whole wave with
     // ceil(EP / 64) experts per lane
-    constexpr int NW = WE * WT, GW = SMALL ? 16 : (EP <= 32 ? 32 : 64), TPW = 64 / GW;
+    // (the lane-group width is part of the canonical summation order of the softmax: it follows
+    // from the padded expert count alone, never from the logit engine)
+    constexpr int NW = WE * WT, GW = EP <= 16 ? 16 : (EP <= 32 ? 32 : 64), TPW = 64 / GW;
     constexpr int EJ = (EP + GW - 1) / GW;
     for (int tb = wave * TPW; tb < BT; tb += NW * TPW) {
         if (t0 + tb >= n) break;
@@ -457,16 +462,29 @@ extern "C" int moe_router(const void* x, const void* w_gate, const float* bias, 
     }
     hipStream_t st = as_stream(stream);
     const int E = p.n_experts;
-    // few tokens: one wave per workgroup so that the (sequential-in-k) work spreads over more CUs
-    const bool few = p.n_tokens <= 64 * 256;
+    // Few tokens are few workgroups, and a workgroup cannot hide the 64-cycle latency of the 32x32
+    // chain: the 4x4 engine with 16 experts per wave then wins although it reads 8x the LDS operand
+    // bytes per MAC.  Measured (h = 2048, 64 experts): 0.10 vs 0.17 ms up to 16k tokens, 0.24 vs 0.26 ms
+    // at 64k, 0.45 vs 0.43 ms at 128k; 160 experts, h = 5120, <= 4k tokens: 0.33 vs 0.45 ms.
+    const bool few = p.n_tokens <= 64 * 1024;       // up to 64 experts
+    const bool few_big = p.n_tokens <= 4096;        // more experts: one workgroup of up to 16 waves per 64 tokens
     if (E <= 4) return launch<true, 1, 1, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
     if (E <= 8) return launch<true, 2, 1, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
     if (E <= 16) return launch<true, 4, 1, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    if (E <= 32) return few ? launch<false, 1, 1, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st)
+    if (E <= 32) return few ? launch<true, 4, 2, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st)
                             : launch<false, 1, 1, 4>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    if (E <= 64) return launch<false, 1, 2, 2>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    if (few && E <= 48) return launch<true, 4, 3, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    if (E <= 64) return few ? launch<true, 4, 4, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st)
+                            : launch<false, 1, 2, 2>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
     // more than 64 experts: one wave per 32 experts (one MFMA per k and wave, no padding beyond
     // the next multiple of 32) measured 10-25 % faster than half as many waves with two MFMAs each
+    if (few_big) {
+        if (E <= 96) return launch<true, 4, 6, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+        if (E <= 128) return launch<true, 4, 8, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+        if (E <= 160) return launch<true, 4, 10, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+        if (E <= 192) return launch<true, 4, 12, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+        return launch<true, 4, 16, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    }
     if (E <= 96) return launch<false, 1, 3, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
     if (E <= 128) return launch<false, 1, 4, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
     if (E <= 160) return launch<false, 1, 5, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);

@@ -126,15 +126,21 @@ def test_router_and_dispatch_golden_fixtures():
 def test_every_expert_count_bracket(E):
     """One case per kernel instantiation (and an odd count inside it): greedy softmax routing and,
     where the count allows groups, sigmoid group-limited routing; logits, indices and weights
-    bit-for-bit.  n = 150 covers two full 64-token tiles and a ragged one; n = 16500 takes the
-    many-token instantiation of the E <= 32 bracket."""
+    bit-for-bit.  n = 150 covers two full 64-token tiles and a ragged one and takes the few-token
+    (4x4 MFMA) engine of every bracket; n = 4100 (more than 64 experts) and n = 65600 (up to 64) take
+    the many-token (32x32 MFMA) engine of the same bracket."""
     print(f"router bracket E={E}", flush=True)
     k = min(6, E)
     g = torch.Generator().manual_seed(E)
     specs = [(O.RouterSpec.deepseek_v2(E, k, "greedy", scale=1.0), False)]
     if E % 4 == 0 and E >= 16:
         specs.append((O.RouterSpec.deepseek_v3(E, k, 4, 2, True, 2.5), True))
-    for n, h in ((150, 136), (16500, 16)) if E in (17, 32) else ((150, 136),):
+    shapes = [(150, 136)]
+    if E > 64:
+        shapes.append((4100, 16))
+    elif E in (17, 32, 33, 64):
+        shapes.append((65600, 16))
+    for n, h in shapes:
         x = torch.randn(n, h, generator=g).to(torch.bfloat16)
         wg = (torch.randn(E, h, generator=g) * 0.1).to(torch.bfloat16)
         for spec, has_bias in specs:
