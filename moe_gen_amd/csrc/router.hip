@@ -233,16 +233,19 @@ __device__ void route_token(const float* row, const float* __restrict__ bias, co
 // Two logit engines share the kernel:
 //  SMALL == false: v_mfma_f32_32x32x1_2b_f32.  NEB: 32-expert MFMA blocks per wave (1 or 2);
 //                  WE / WT: waves along experts / tokens.
-//  SMALL == true : v_mfma_f32_4x4x1_16b_f32: one instruction is 64 tokens x 4 experts in 8 cycles, so
-//                  nothing is padded to 32 experts and the sequential-in-k dependency chain is 8x
-//                  shorter.  NEB = groups of 4 experts per wave (1..4), WE waves along experts.  Used
-//                  for E <= 16 (Mixtral's 8 experts) and, with few tokens, up to 64 experts: a handful
-//                  of workgroups cannot hide the 64-cycle latency of the 32x32 chain, and 16 experts
-//                  per wave spread the work over twice as many waves (it reads 8x the LDS operand
-//                  bytes per MAC, which is why many tokens stay on the 32x32 engine).
+//  SMALL == true : v_mfma_f32_4x4x1_16b_f32: 16 independent 4x4 blocks in 8 cycles, so nothing is
+//                  padded to 32 experts and the sequential-in-k dependency chain is 8x shorter.  The
+//                  blocks are TG groups of 4 tokens x 16/TG groups of 4 experts: TG = 16 is 64 tokens
+//                  x 4 experts per instruction, TG = 4 is 16 x 16, TG = 1 is 4 x 64; a workgroup owns
+//                  4*TG tokens.  NEB instructions per k and wave, WE waves along experts.  Used for
+//                  E <= 16 (Mixtral's 8 experts) and for few tokens: a handful of workgroups cannot hide
+//                  the 64-cycle latency of the 32x32 chain, and fewer tokens per workgroup spread the
+//                  chains over more CUs (it reads 8x the LDS operand bytes per MAC, which is why many
+//                  tokens stay on the 32x32 engine).
+//  GW: lanes per token in the selection (16, 32 or 64 for E <= 16, <= 32, more).
 // Global loads run two k-stages ahead in registers (two register sets, loop unrolled by two), which
 // is what hides the load latency when only a few workgroups exist (small token counts).
-template <bool SMALL, int NEB, int WE, int WT>
+template <bool SMALL, int TG, int NEB, int WE, int WT, int GW>
 __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ wg, const float* __restrict__ bias,
     moe_router_params p, int32_t* __restrict__ topk_idx, float* __restrict__ topk_w,
@@ -250,8 +253,12 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     constexpr int KC = SMALL ? 64 : 32;  // k elements per LDS stage
     constexpr int LDK = KC + 4;          // padded fp32 row stride: conflict-free 16-byte reads
     constexpr int NT = 64 * WE * WT;  // threads
-    constexpr int BT = 64 * WT;       // tokens per block
-    constexpr int EP = SMALL ? 4 * NEB * WE : 32 * NEB * WE;  // padded experts per block
+    // SMALL: the 16 blocks of an instruction are TG groups of 4 tokens x EG groups of 4 experts
+    constexpr int EG = SMALL ? 16 / TG : 1;
+    constexpr int BT = SMALL ? 4 * TG * WT : 64 * WT;          // tokens per block
+    constexpr int EPW = SMALL ? 4 * EG * NEB : 32 * NEB;       // experts per wave
+    constexpr int EP = EPW * WE;                                // padded experts per block
+    static_assert(!SMALL || (TG * EG == 16 && WT == 1), "4x4 engine: 16 blocks per instruction, one wave along tokens");
     constexpr int XCH = BT * (KC / 8), WCH = EP * (KC / 8);  // 16-byte chunks per stage
     constexpr int XPT = (XCH + NT - 1) / NT, WPT = (WCH + NT - 1) / NT;
     constexpr int TILE_F = (BT + EP) * LDK, LOGIT_F = BT * EP;
@@ -315,8 +322,10 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     f32x4 acc4[SMALL ? NEB : 1];            // SMALL == true: group j = experts 4j .. 4j+3
 #pragma unroll
     for (int j = 0; j < (SMALL ? NEB : 1); ++j) acc4[j] = f32x4{0, 0, 0, 0};
-    const float* a_row = Xs + (wt * 64 + lane) * LDK;
-    const float* b0_row = SMALL ? Ws + (we * 4 * NEB + (lane & 3)) * LDK
+    // 4x4 engine: lane l feeds block l/4 = (token group tg, expert group eg), row / column l%4
+    const int tg = (lane >> 2) / EG, eg = (lane >> 2) % EG;
+    const float* a_row = SMALL ? Xs + (4 * tg + (lane & 3)) * LDK : Xs + (wt * 64 + lane) * LDK;
+    const float* b0_row = SMALL ? Ws + (we * EPW + 4 * eg + (lane & 3)) * LDK
                                 : Ws + (NEB == 2 ? (we * 64 + lane) : (we * 32 + (lane & 31))) * LDK;
     const float* b1_row = Ws + (we * 64 + (lane ^ 32)) * LDK;  // only read when !SMALL && NEB == 2
 
@@ -326,7 +335,7 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
         a = *reinterpret_cast<const f32x4*>(a_row + k4 * 4);
         if (SMALL) {
 #pragma unroll
-            for (int j = 0; j < NEB; ++j) b[j] = *reinterpret_cast<const f32x4*>(b0_row + j * 4 * LDK + k4 * 4);
+            for (int j = 0; j < NEB; ++j) b[j] = *reinterpret_cast<const f32x4*>(b0_row + j * 4 * EG * LDK + k4 * 4);
         } else {
             b[0] = *reinterpret_cast<const f32x4*>(b0_row + k4 * 4);
             if (NEB == 2) b[1] = *reinterpret_cast<const f32x4*>(b1_row + k4 * 4);
@@ -377,11 +386,11 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     // accumulators -> LDS logits[token][expert]
     float* lg = lds;
     if (SMALL) {
-        // register i of lane l of group j: token 4*(l/4) + i, expert 4*j + l%4
+        // register i of lane l of instruction j: token 4*tg + i, expert 4*EG*j + 4*eg + l%4 of the wave's
 #pragma unroll
         for (int j = 0; j < NEB; ++j)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) lg[(wt * 64 + 4 * (lane >> 2) + i) * EP + we * 4 * NEB + 4 * j + (lane & 3)] = acc4[j][i];
+            for (int i = 0; i < 4; ++i) lg[(4 * tg + i) * EP + we * EPW + 4 * EG * j + 4 * eg + (lane & 3)] = acc4[j][i];
     } else {
         // in block b of the 2-block MFMA result, register 16*b+i of lane l is row
         // 8*(i/4) + 4*(l/32) + i%4, column l%32
@@ -403,11 +412,11 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     }
     __syncthreads();
 
-    // selection, a lane group per token: 16 lanes for E <= 16, 32 for E <= 32, else the whole wave with
-    // ceil(EP / 64) experts per lane
+    // selection, a lane group per token: GW = 16 lanes for E <= 16, 32 for E <= 32, else the whole wave,
+    // with ceil(EP / GW) experts per lane
     // (the lane-group width is part of the canonical summation order of the softmax: it follows
-    // from the padded expert count alone, never from the logit engine)
-    constexpr int NW = WE * WT, GW = EP <= 16 ? 16 : (EP <= 32 ? 32 : 64), TPW = 64 / GW;
+    // from the expert count alone, never from the logit engine or its padding)
+    constexpr int NW = WE * WT, TPW = 64 / GW;
     constexpr int EJ = (EP + GW - 1) / GW;
     for (int tb = wave * TPW; tb < BT; tb += NW * TPW) {
         if (t0 + tb >= n) break;
@@ -420,12 +429,12 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     }
 }
 
-template <bool SMALL, int NEB, int WE, int WT>
+template <bool SMALL, int TG, int NEB, int WE, int WT, int GW>
 int launch(const void* x, const void* w, const float* bias, const moe_router_params& p, int32_t* idx,
            float* tw, float* lo, hipStream_t st) {
-    constexpr int BT = 64 * WT;
+    constexpr int BT = SMALL ? 4 * TG * WT : 64 * WT;
     dim3 grid((p.n_tokens + BT - 1) / BT), block(64 * WE * WT);
-    hipLaunchKernelGGL((router_kernel<SMALL, NEB, WE, WT>), grid, block, 0, st, (const uint16_t*)x,
+    hipLaunchKernelGGL((router_kernel<SMALL, TG, NEB, WE, WT, GW>), grid, block, 0, st, (const uint16_t*)x,
                        (const uint16_t*)w, bias, p, idx, tw, lo);
     MOE_HIP_CHECK(hipGetLastError());
     return MOE_OK;
@@ -461,34 +470,56 @@ extern "C" int moe_router(const void* x, const void* w_gate, const float* bias, 
                     "moe_router: noaux_tc needs at least 2 experts per group");
     }
     hipStream_t st = as_stream(stream);
-    const int E = p.n_experts;
-    // Few tokens are few workgroups, and a workgroup cannot hide the 64-cycle latency of the 32x32
-    // chain: the 4x4 engine with 16 experts per wave then wins although it reads 8x the LDS operand
-    // bytes per MAC.  Measured (h = 2048, 64 experts): 0.10 vs 0.17 ms up to 16k tokens, 0.24 vs 0.26 ms
-    // at 64k, 0.45 vs 0.43 ms at 128k; 160 experts, h = 5120, <= 4k tokens: 0.33 vs 0.45 ms.
-    const bool few = p.n_tokens <= 64 * 1024;       // up to 64 experts
-    const bool few_big = p.n_tokens <= 4096;        // more experts: one workgroup of up to 16 waves per 64 tokens
-    if (E <= 4) return launch<true, 1, 1, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    if (E <= 8) return launch<true, 2, 1, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    if (E <= 16) return launch<true, 4, 1, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    if (E <= 32) return few ? launch<true, 4, 2, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st)
-                            : launch<false, 1, 1, 4>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    if (few && E <= 48) return launch<true, 4, 3, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    if (E <= 64) return few ? launch<true, 4, 4, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st)
-                            : launch<false, 1, 2, 2>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    // more than 64 experts: one wave per 32 experts (one MFMA per k and wave, no padding beyond
-    // the next multiple of 32) measured 10-25 % faster than half as many waves with two MFMAs each
-    if (few_big) {
-        if (E <= 96) return launch<true, 4, 6, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-        if (E <= 128) return launch<true, 4, 8, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-        if (E <= 160) return launch<true, 4, 10, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-        if (E <= 192) return launch<true, 4, 12, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-        return launch<true, 4, 16, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    const int E = p.n_experts, n = p.n_tokens;
+#define MOE_ROUTE(SMALL, TG, NEB, WE, WT, GW) \
+    return launch<SMALL, TG, NEB, WE, WT, GW>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st)
+    // The 4x4 engine's 16 blocks per instruction are laid out as 64 tokens x 4 experts, 16 x 16 or
+    // 4 x 64: the fewer tokens a launch has, the fewer go to a workgroup, so that the sequential-in-k
+    // chains run on as many CUs as possible; many tokens take the 32x32 engine (an eighth of the LDS
+    // operand bytes per MAC).  The switch points are measured ones (ms, h = 2048 / 5120 / 7168):
+    //   64 experts    4096 tokens: 16x16 0.040, 64x4 0.097;  24576: 0.122, 0.148;  32768: 0.157, 0.153;
+    //                 131072: 64x4 0.45, 32x32 0.43
+    //   8 experts    32768 tokens: 16x16 0.093, 64x4 0.104;  65536: 0.174, 0.144
+    //   160 experts   1024 tokens: 4x64 0.115, 16x16 0.131, 64x4 0.335;  8192: 16x16 0.250, 32x32 0.468;
+    //                 12288: 0.374, 0.479
+    //   256 experts   1024 tokens: 4x64 0.165, 16x16 0.231, 64x4 0.583;  8192: 16x16 0.519, 32x32 0.657;
+    //                 12288: 0.775, 0.683
+    if (E <= 64) {
+        if (n <= (E <= 32 ? 32768 : 24576)) {   // 16 tokens per workgroup, 16 experts per wave
+            if (E <= 16) MOE_ROUTE(true, 4, 1, 1, 1, 16);
+            if (E <= 32) MOE_ROUTE(true, 4, 1, 2, 1, 32);
+            if (E <= 48) MOE_ROUTE(true, 4, 1, 3, 1, 64);
+            MOE_ROUTE(true, 4, 1, 4, 1, 64);
+        }
+        if (E <= 4) MOE_ROUTE(true, 16, 1, 1, 1, 16);   // 64 tokens per workgroup, 4 .. 16 experts per wave
+        if (E <= 8) MOE_ROUTE(true, 16, 2, 1, 1, 16);
+        if (E <= 16) MOE_ROUTE(true, 16, 4, 1, 1, 16);
+        if (n <= 65536) {
+            if (E <= 32) MOE_ROUTE(true, 16, 4, 2, 1, 32);
+            if (E <= 48) MOE_ROUTE(true, 16, 4, 3, 1, 64);
+            MOE_ROUTE(true, 16, 4, 4, 1, 64);
+        }
+        if (E <= 32) MOE_ROUTE(false, 16, 1, 1, 4, 32);
+        MOE_ROUTE(false, 16, 1, 2, 2, 64);
     }
-    if (E <= 96) return launch<false, 1, 3, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    if (E <= 128) return launch<false, 1, 4, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    if (E <= 160) return launch<false, 1, 5, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    if (E <= 192) return launch<false, 1, 6, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    if (E <= 224) return launch<false, 1, 7, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
-    return launch<false, 1, 8, 1>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    if (n <= 1024 && E > 128) {                 // 4 tokens per workgroup, 64 experts per wave
+        if (E <= 192) MOE_ROUTE(true, 1, 1, 3, 1, 64);
+        MOE_ROUTE(true, 1, 1, 4, 1, 64);
+    }
+    if (n <= 8192) {                            // 16 tokens per workgroup, 16 experts per wave
+        if (E <= 96) MOE_ROUTE(true, 4, 1, 6, 1, 64);
+        if (E <= 128) MOE_ROUTE(true, 4, 1, 8, 1, 64);
+        if (E <= 160) MOE_ROUTE(true, 4, 1, 10, 1, 64);
+        if (E <= 192) MOE_ROUTE(true, 4, 1, 12, 1, 64);
+        MOE_ROUTE(true, 4, 1, 16, 1, 64);
+    }
+    // many tokens, more than 64 experts: one wave per 32 experts (one MFMA per k and wave, no padding
+    // beyond the next multiple of 32) measured 10-25 % faster than half as many waves with two MFMAs each
+    if (E <= 96) MOE_ROUTE(false, 16, 1, 3, 1, 64);
+    if (E <= 128) MOE_ROUTE(false, 16, 1, 4, 1, 64);
+    if (E <= 160) MOE_ROUTE(false, 16, 1, 5, 1, 64);
+    if (E <= 192) MOE_ROUTE(false, 16, 1, 6, 1, 64);
+    if (E <= 224) MOE_ROUTE(false, 16, 1, 7, 1, 64);
+    MOE_ROUTE(false, 16, 1, 8, 1, 64);
+#undef MOE_ROUTE
 }

@@ -126,9 +126,11 @@ def test_router_and_dispatch_golden_fixtures():
 def test_every_expert_count_bracket(E):
     """One case per kernel instantiation (and an odd count inside it): greedy softmax routing and,
     where the count allows groups, sigmoid group-limited routing; logits, indices and weights
-    bit-for-bit.  n = 150 covers two full 64-token tiles and a ragged one and takes the few-token
-    (4x4 MFMA) engine of every bracket; n = 4100 (more than 64 experts) and n = 65600 (up to 64) take
-    the many-token (32x32 MFMA) engine of the same bracket."""
+    bit-for-bit.  The token count picks the logit engine and its block layout inside a bracket:
+    150 tokens (full tiles and a ragged one) the 4x4 MFMA engine with 16 tokens per workgroup, or
+    with 4 above 128 experts; 4100 tokens (more than 128 experts) 16 per workgroup; 8200 tokens
+    (more than 64 experts) the 32x32 MFMA engine; up to 64 experts 33000 tokens the 4x4 engine with
+    64 tokens per workgroup and 65600 the 32x32 engine (always 4x4 up to 16 experts)."""
     print(f"router bracket E={E}", flush=True)
     k = min(6, E)
     g = torch.Generator().manual_seed(E)
@@ -137,9 +139,13 @@ def test_every_expert_count_bracket(E):
         specs.append((O.RouterSpec.deepseek_v3(E, k, 4, 2, True, 2.5), True))
     shapes = [(150, 136)]
     if E > 64:
-        shapes.append((4100, 16))
-    elif E in (17, 32, 33, 64):
-        shapes.append((65600, 16))
+        shapes.append((8200, 16))
+        if E > 128:
+            shapes.append((4100, 16))
+    else:
+        shapes.append((33000, 16))
+        if E in (17, 32, 33, 64):
+            shapes.append((65600, 16))
     for n, h in shapes:
         x = torch.randn(n, h, generator=g).to(torch.bfloat16)
         wg = (torch.randn(E, h, generator=g) * 0.1).to(torch.bfloat16)
