@@ -156,3 +156,44 @@ def test_every_expert_count_bracket(E):
             assert np.array_equal(lg.view(np.uint32), ol.view(np.uint32)), (E, n, spec.method)
             assert np.array_equal(idx, oi), (E, n, spec.method)
             assert np.array_equal(w.view(np.uint32), ow.view(np.uint32)), (E, n, spec.method)
+
+
+def test_router_random_shapes_at_switch_points():
+    """Seeded random rules (expert count, top-k, family, groups) at token counts on both sides of
+    every switch point of the logit engine's dispatch, bit-for-bit against the oracle."""
+    import random
+    rng = random.Random(7)
+    edges = [1, 3, 4, 5, 15, 16, 17, 63, 64, 65, 1023, 1024, 1025, 8191, 8192, 8193, 24576, 24577, 32768,
+             32769, 65536, 65537]
+    for it in range(40):
+        E = rng.choice([1, 3, 7, 9, 16, 20, 31, 32, 40, 50, 64, 72, 96, 120, 129, 160, 190, 208, 240, 256])
+        k = rng.randint(1, min(E, 8))
+        fam = rng.choice(["v2_greedy", "v2_group", "v3", "mixtral"])
+        divs = [g for g in (2, 4, 8, 16) if E % g == 0 and E // g >= 2]
+        if fam in ("v2_group", "v3") and not divs:
+            fam = "v2_greedy"
+        has_bias = False
+        if fam == "v2_greedy":
+            spec = O.RouterSpec.deepseek_v2(E, k, "greedy", scale=rng.choice([1.0, 16.0]), norm=rng.random() < 0.5)
+        elif fam == "mixtral":
+            spec = O.RouterSpec.mixtral(E, k)
+        else:
+            G = rng.choice(divs)
+            Kg = rng.randint(1, G)
+            k = min(k, Kg * (E // G))
+            if fam == "v2_group":
+                spec = O.RouterSpec.deepseek_v2(E, k, "group_limited_greedy", G, Kg, rng.random() < 0.5, 16.0)
+            else:
+                spec, has_bias = O.RouterSpec.deepseek_v3(E, k, G, Kg, rng.random() < 0.7, 2.5), True
+        n = rng.choice(edges)
+        h = 8 * rng.randint(1, 12)
+        print(f"router random case {it}: E={E} k={k} {fam} n={n} h={h}", flush=True)
+        g = torch.Generator().manual_seed(1000 + it)
+        x = torch.randn(n, h, generator=g).to(torch.bfloat16)
+        wg = (torch.randn(E, h, generator=g) * 0.1).to(torch.bfloat16)
+        bias = (torch.randn(E, generator=g) * 0.01) if has_bias else None
+        idx, w, lg = gpu_router(x, wg, bias, spec)
+        oi, ow, ol = O.router(bits(x), bits(wg), None if bias is None else bias.numpy(), spec)
+        assert np.array_equal(lg.view(np.uint32), ol.view(np.uint32)), (it, E, n, fam)
+        assert np.array_equal(idx, oi), (it, E, n, fam)
+        assert np.array_equal(w.view(np.uint32), ow.view(np.uint32)), (it, E, n, fam)
