@@ -22,9 +22,12 @@ constexpr int MAX_K = 16;
 
 // KB: source rows whose 16-byte chunks a lane requests back to back before it starts adding (the
 // sum itself stays in slot order).  The kernel is bound by HBM latency x bytes in flight, and one
-// outstanding load per lane is too few.
+// outstanding load per lane is too few.  The block has one lane per chunk of the row where that
+// fits (up to 1024 threads), so a token's loads all leave at once.  Expert outputs are read once and
+// the result is not read again here: both go past the caches non-temporally (measured on 65536 x 8
+// rows of 7168: 1.90 -> 1.70 ms; 32768 x 6 of 5120: 0.54 -> 0.46 ms).
 template <int MODE, int KB>
-__global__ __launch_bounds__(256) void combine_kernel(const u32x4* __restrict__ y, const int32_t* __restrict__ pos,
+__global__ __launch_bounds__(1024) void combine_kernel(const u32x4* __restrict__ y, const int32_t* __restrict__ pos,
                                                       const int32_t* __restrict__ topk_idx,
                                                       const float* __restrict__ topk_w, const u32x4* __restrict__ shared,
                                                       const u32x4* residual, int k, int chunks, u32x4* out) {
@@ -46,15 +49,15 @@ __global__ __launch_bounds__(256) void combine_kernel(const u32x4* __restrict__ 
         s_w[a] = (MODE == MOE_COMBINE_F32) ? w : round_to_bf16(w);
     }
     __syncthreads();
-    for (int c = threadIdx.x; c < chunks; c += 256) {
+    for (int c = threadIdx.x; c < chunks; c += blockDim.x) {
         float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         u32x4 sh = {0, 0, 0, 0}, res = {0, 0, 0, 0};
-        if (shared) sh = shared[(size_t)t * chunks + c];
-        if (residual) res = residual[(size_t)t * chunks + c];   // may alias out: read before this thread writes
+        if (shared) sh = __builtin_nontemporal_load(&shared[(size_t)t * chunks + c]);
+        if (residual) res = __builtin_nontemporal_load(&residual[(size_t)t * chunks + c]);   // may alias out: read before this thread writes
         for (int a0 = 0; a0 < k; a0 += KB) {
         u32x4 vb[KB];
 #pragma unroll
-        for (int b = 0; b < KB; ++b) vb[b] = y[(size_t)s_row[min(a0 + b, k - 1)] * chunks + c];   // past k: the last row again
+        for (int b = 0; b < KB; ++b) vb[b] = __builtin_nontemporal_load(&y[(size_t)s_row[min(a0 + b, k - 1)] * chunks + c]);   // past k: the last row again
 #pragma unroll
         for (int b = 0; b < KB; ++b) {
             if (a0 + b >= k) break;
@@ -96,7 +99,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const u32x4* __restrict__ 
                 o[i] = lo | (hi << 16);
             }
         }
-        out[(size_t)t * chunks + c] = o;
+        __builtin_nontemporal_store(o, &out[(size_t)t * chunks + c]);
     }
 }
 
@@ -117,12 +120,14 @@ int combine_impl(const void* y, const int32_t* pos, const int32_t* topk_idx, con
     MOE_REQUIRE(mode != MOE_COMBINE_BF16_SEQ || topk_idx, "%s: topk_idx is required for MOE_COMBINE_BF16_SEQ", who);
     MOE_REQUIRE(out != y && out != shared, "%s: out must not alias y or shared", who);
     hipStream_t st = as_stream(stream);
-    dim3 grid(n_tokens), block(256);
+    const int chunks = hidden / 8;
+    const int passes = (chunks + 1023) / 1024;                       // 1 up to hidden = 8192
+    const int threads = (((chunks + passes - 1) / passes + 63) / 64) * 64;
+    dim3 grid(n_tokens), block(threads);
     const u32x4* yv = static_cast<const u32x4*>(y);
     const u32x4* sv = static_cast<const u32x4*>(shared);
     const u32x4* rv = static_cast<const u32x4*>(residual);
     u32x4* ov = static_cast<u32x4*>(out);
-    const int chunks = hidden / 8;
 #define MOE_LAUNCH_COMBINE(M, B) \
     hipLaunchKernelGGL((combine_kernel<M, B>), grid, block, 0, st, yv, pos, topk_idx, topk_w, sv, rv, top_k, chunks, ov)
 #define MOE_LAUNCH_COMBINE_K(M)                          \
