@@ -66,7 +66,8 @@ def test_dispatch_full_size_properties():
 
 @pytest.mark.parametrize("mode", [0, 1, 2])
 @pytest.mark.parametrize("n,k,h,shared", [(1, 1, 8, False), (50, 2, 64, False), (257, 6, 2048, True),
-                                          (100, 8, 7168, True)])
+                                          (100, 8, 7168, True), (33, 3, 5120, True), (9, 4, 8200, True),
+                                          (5, 6, 16384, False)])   # 8200, 16384: more than one pass per block
 def test_combine_bit_exact(mode, n, k, h, shared):
     from moe_gen_amd import ops
     print(f"combine mode={mode} n={n} k={k} h={h} shared={shared}", flush=True)
