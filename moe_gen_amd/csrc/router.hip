@@ -243,9 +243,13 @@ __device__ void route_token(const float* row, const float* __restrict__ bias, co
 //                  chains over more CUs (it reads 8x the LDS operand bytes per MAC, which is why many
 //                  tokens stay on the 32x32 engine).
 //  GW: lanes per token in the selection (16, 32 or 64 for E <= 16, <= 32, more).
+//  NX (32x32 engine only): groups of 4 more experts that each wave adds with 4x4 instructions on the
+//                  same token operand.  Both instructions cost 2 cycles per expert and k, so 160
+//                  experts as 4 waves x (32 + 8) load the four SIMDs evenly (80 cycles per k each),
+//                  where 5 waves x 32 put two waves on one SIMD (128 cycles, as slow as 256 experts).
 // Global loads run two k-stages ahead in registers (two register sets, loop unrolled by two), which
 // is what hides the load latency when only a few workgroups exist (small token counts).
-template <bool SMALL, int TG, int NEB, int WE, int WT, int GW>
+template <bool SMALL, int TG, int NEB, int WE, int WT, int GW, int NX = 0>
 __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ wg, const float* __restrict__ bias,
     moe_router_params p, int32_t* __restrict__ topk_idx, float* __restrict__ topk_w,
@@ -256,7 +260,8 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     // SMALL: the 16 blocks of an instruction are TG groups of 4 tokens x EG groups of 4 experts
     constexpr int EG = SMALL ? 16 / TG : 1;
     constexpr int BT = SMALL ? 4 * TG * WT : 64 * WT;          // tokens per block
-    constexpr int EPW = SMALL ? 4 * EG * NEB : 32 * NEB;       // experts per wave
+    constexpr int EPW = SMALL ? 4 * EG * NEB : 32 * NEB + 4 * NX;   // experts per wave
+    static_assert(NX == 0 || (!SMALL && NEB == 1), "extra 4-expert groups go with one 32x32 block per wave");
     constexpr int EP = EPW * WE;                                // padded experts per block
     static_assert(!SMALL || (TG * EG == 16 && WT == 1), "4x4 engine: 16 blocks per instruction, one wave along tokens");
     constexpr int XCH = BT * (KC / 8), WCH = EP * (KC / 8);  // 16-byte chunks per stage
@@ -319,18 +324,20 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     };
 
     f32x32 acc0 = {0}, acc1 = {0};          // SMALL == false
-    f32x4 acc4[SMALL ? NEB : 1];            // SMALL == true: group j = experts 4j .. 4j+3
+    constexpr int N4 = SMALL ? NEB : (NX > 0 ? NX : 1);
+    f32x4 acc4[N4];                         // SMALL: group j = experts 4j .. 4j+3; else the NX extra groups
 #pragma unroll
-    for (int j = 0; j < (SMALL ? NEB : 1); ++j) acc4[j] = f32x4{0, 0, 0, 0};
+    for (int j = 0; j < N4; ++j) acc4[j] = f32x4{0, 0, 0, 0};
     // 4x4 engine: lane l feeds block l/4 = (token group tg, expert group eg), row / column l%4
     const int tg = (lane >> 2) / EG, eg = (lane >> 2) % EG;
     const float* a_row = SMALL ? Xs + (4 * tg + (lane & 3)) * LDK : Xs + (wt * 64 + lane) * LDK;
     const float* b0_row = SMALL ? Ws + (we * EPW + 4 * eg + (lane & 3)) * LDK
-                                : Ws + (NEB == 2 ? (we * 64 + lane) : (we * 32 + (lane & 31))) * LDK;
+                                : Ws + (NEB == 2 ? (we * 64 + lane) : (we * EPW + (lane & 31))) * LDK;
+    const float* bx_row = Ws + (we * EPW + 32 + (lane & 3)) * LDK;   // only read when NX > 0
     const float* b1_row = Ws + (we * 64 + (lane ^ 32)) * LDK;  // only read when !SMALL && NEB == 2
 
     // operands of k..k+3 are read (16 bytes per lane) one step ahead of the MFMAs that use them
-    constexpr int NB4 = SMALL ? NEB : 2;
+    constexpr int NB4 = SMALL ? NEB : 2 + NX;
     auto read_ops = [&](int k4, f32x4& a, f32x4 (&b)[NB4]) {
         a = *reinterpret_cast<const f32x4*>(a_row + k4 * 4);
         if (SMALL) {
@@ -339,6 +346,8 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
         } else {
             b[0] = *reinterpret_cast<const f32x4*>(b0_row + k4 * 4);
             if (NEB == 2) b[1] = *reinterpret_cast<const f32x4*>(b1_row + k4 * 4);
+#pragma unroll
+            for (int j = 0; j < NX; ++j) b[2 + j] = *reinterpret_cast<const f32x4*>(bx_row + j * 4 * LDK + k4 * 4);
         }
     };
     auto multiply_stage = [&]() {
@@ -357,6 +366,9 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
                 } else {
                     acc0 = __builtin_amdgcn_mfma_f32_32x32x1f32(a[k4 & 1][kk], b[k4 & 1][0][kk], acc0, 0, 0, 0);
                     if (NEB == 2) acc1 = __builtin_amdgcn_mfma_f32_32x32x1f32(a[k4 & 1][kk], b[k4 & 1][1][kk], acc1, 0, 0, 0);
+#pragma unroll
+                    for (int j = 0; j < NX; ++j)
+                        acc4[j] = __builtin_amdgcn_mfma_f32_4x4x1f32(a[k4 & 1][kk], b[k4 & 1][2 + j][kk], acc4[j], 0, 0, 0);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -405,10 +417,15 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
                     lg[tl * EP + e0] = acc0[16 * b + i];
                     lg[tl * EP + e1] = acc1[16 * b + i];
                 } else {
-                    lg[tl * EP + we * 32 + (lane & 31)] = acc0[16 * b + i];
+                    lg[tl * EP + we * EPW + (lane & 31)] = acc0[16 * b + i];
                 }
             }
         }
+        // the extra groups: register i of lane l of group j is token 4*(l/4) + i, expert 32 + 4*j + l%4 of the wave's
+#pragma unroll
+        for (int j = 0; j < NX; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) lg[(wt * 64 + 4 * (lane >> 2) + i) * EP + we * EPW + 32 + 4 * j + (lane & 3)] = acc4[j][i];
     }
     __syncthreads();
 
@@ -429,12 +446,12 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     }
 }
 
-template <bool SMALL, int TG, int NEB, int WE, int WT, int GW>
+template <bool SMALL, int TG, int NEB, int WE, int WT, int GW, int NX = 0>
 int launch(const void* x, const void* w, const float* bias, const moe_router_params& p, int32_t* idx,
            float* tw, float* lo, hipStream_t st) {
     constexpr int BT = SMALL ? 4 * TG * WT : 64 * WT;
     dim3 grid((p.n_tokens + BT - 1) / BT), block(64 * WE * WT);
-    hipLaunchKernelGGL((router_kernel<SMALL, TG, NEB, WE, WT, GW>), grid, block, 0, st, (const uint16_t*)x,
+    hipLaunchKernelGGL((router_kernel<SMALL, TG, NEB, WE, WT, GW, NX>), grid, block, 0, st, (const uint16_t*)x,
                        (const uint16_t*)w, bias, p, idx, tw, lo);
     MOE_HIP_CHECK(hipGetLastError());
     return MOE_OK;
@@ -515,11 +532,21 @@ extern "C" int moe_router(const void* x, const void* w_gate, const float* bias, 
     }
     // many tokens, more than 64 experts: one wave per 32 experts (one MFMA per k and wave, no padding
     // beyond the next multiple of 32) measured 10-25 % faster than half as many waves with two MFMAs each
+#define MOE_ROUTE_X(WE, NX) \
+    return launch<false, 16, 1, WE, 1, 64, NX>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st)
     if (E <= 96) MOE_ROUTE(false, 16, 1, 3, 1, 64);
     if (E <= 128) MOE_ROUTE(false, 16, 1, 4, 1, 64);
-    if (E <= 160) MOE_ROUTE(false, 16, 1, 5, 1, 64);
-    if (E <= 192) MOE_ROUTE(false, 16, 1, 6, 1, 64);
+    // Between 4 and 8 waves' worth of experts: 4 waves x (32 + 4 NX) keep the four SIMDs evenly loaded,
+    // where 5, 6 or 7 waves of 32 put two waves on one SIMD and run as slowly as 8.  Measured, 32768
+    // tokens, h = 5120 (ms): 144 experts 0.72 -> 0.56, 160: 0.77 -> 0.67 (131072 tokens: 2.93 -> 2.11),
+    // 176: 0.77 -> 0.64, 192: 0.77 -> 0.68, 208: 0.79 -> 0.74; from 209 on the 8 (7) waves are as fast.
+    if (E <= 144) MOE_ROUTE_X(4, 1);
+    if (E <= 160) MOE_ROUTE_X(4, 2);
+    if (E <= 176) MOE_ROUTE_X(4, 3);
+    if (E <= 192) MOE_ROUTE_X(4, 4);
+    if (E <= 208) MOE_ROUTE_X(4, 5);
     if (E <= 224) MOE_ROUTE(false, 16, 1, 7, 1, 64);
     MOE_ROUTE(false, 16, 1, 8, 1, 64);
+#undef MOE_ROUTE_X
 #undef MOE_ROUTE
 }

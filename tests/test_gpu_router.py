@@ -129,7 +129,7 @@ def test_every_expert_count_bracket(E):
     bit-for-bit.  The token count picks the logit engine and its block layout inside a bracket:
     150 tokens (full tiles and a ragged one) the 4x4 MFMA engine with 16 tokens per workgroup, or
     with 4 above 128 experts; 4100 tokens (more than 128 experts) 16 per workgroup; 8200 tokens
-    (more than 64 experts) the 32x32 MFMA engine; up to 64 experts 33000 tokens the 4x4 engine with
+    (more than 64 experts) the 32x32 MFMA engine (129 to 208 experts: with extra 4-expert groups per wave); up to 64 experts 33000 tokens the 4x4 engine with
     64 tokens per workgroup and 65600 the 32x32 engine (always 4x4 up to 16 experts)."""
     print(f"router bracket E={E}", flush=True)
     k = min(6, E)
