@@ -94,13 +94,16 @@ int moe_router(const void* x, const void* w_gate, const float* bias,
  *   offsets   device int32 [E+1]    out  exclusive prefix sum of counts
  *   perm      device int32 [n*k]    out  perm[r] = flat index at sorted row r
  *   pos       device int32 [n*k]    out  pos[flat] = sorted row (inverse of perm)
+ *   row_map   device int32 [n*k]    out  row_map[r] = perm[r] / k, the token behind sorted row r
+ *                                        (what the grouped GEMM's fused gather reads); may be NULL
  *   x         device bf16 [n, h]         may be NULL together with xs
  *   xs        device bf16 [n*k, h]  out  gathered rows, may be NULL
  *   workspace device, at least moe_dispatch_workspace_bytes(n, k, E) bytes
+ * An id outside [0, E) is not counted and owns no sorted row; its pos entry is 0.
  */
 size_t moe_dispatch_workspace_bytes(int32_t n_tokens, int32_t top_k, int32_t n_experts);
 int moe_dispatch(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k, int32_t n_experts,
-                 int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* pos,
+                 int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* pos, int32_t* row_map,
                  const void* x, int32_t hidden, void* xs,
                  void* workspace, size_t workspace_bytes, void* stream);
 
@@ -119,7 +122,11 @@ int moe_dispatch(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k, int32
  *   row_map   device int32 [n_rows] or NULL
  *   w_gate/w_up/w_down   device arrays of E device pointers: Wg_e, Wu_e bf16
  *             [I, h]; Wd_e bf16 [h, I]  (nn.Linear [out, in] layout)
- *   offsets   device int32 [E+1] (as written by moe_dispatch); offsets[E] <= n_rows
+ *   offsets   device int32 [E+1] (as written by moe_dispatch).  Rows are absolute indices into
+ *             act / y / row_map, so a call may cover a sub-range [a, b) of a layer's experts by
+ *             passing offsets + a, the pointer arrays + a and E = b - a (weights handed out in
+ *             waves by a pool smaller than the layer); n_rows must then be at least
+ *             offsets[b] - offsets[a], the rows inside the range
  *   act       device bf16 [n_rows, I]  scratch for a
  *   y         device bf16 [n_rows, h]  out
  *   workspace reserved: the kernels find their tiles from offsets[] on the device and need no
@@ -216,8 +223,8 @@ int moe_combine_residual(const void* y, const int32_t* pos, const int32_t* topk_
  * into HBM slots on a private copy stream.  Replaces, for the weights half,
  * HtoD_Engine::HtoD_Worker (core/HtoD_Engine/HtoD_Engine.cpp:201-268),
  * GPU_Weight_Buffer::{acquireEmptyBuffer, get_weights, releaseBuffer,
- * weights_copy_complete, clear_expert_buffer}
- * (core/GPU_Weight_Buffer/GPU_Weight_Buffer.cpp:146-308) and
+ * weights_copy_complete, clear_expert_buffer, resize_buffer, reset_prefill_buffer}
+ * (core/GPU_Weight_Buffer/GPU_Weight_Buffer.cpp:103-379) and
  * Weights_Storage::get_module_weights_storage (core/Weights_Storage/Weights_Storage.cpp:80).
  * The reference hands slots over through a host condition variable after a
  * stream synchronise; here hand-off is by events: acquire() makes the caller's
@@ -227,7 +234,9 @@ int moe_combine_residual(const void* y, const int32_t* pos, const int32_t* topk_
  * A "module type" is a family of modules sharing one slot shape (the reference's
  * "routed_expert", "shared_expert").  Modules are copied in the cyclic order in
  * which they were added, routing-agnostically, whenever a slot of their type is
- * free -- the policy of the reference's worker loop.
+ * free -- the policy of the reference's worker loop.  A module that is still resident when
+ * its turn comes keeps its place in the cycle and the next non-resident one is copied (the
+ * reference would copy it a second time); in the reference's order of use this never happens.
  */
 typedef struct moe_stager moe_stager;
 
@@ -267,11 +276,44 @@ int moe_stage_set_policy(moe_stager* s, int32_t type, int32_t policy);
 int moe_stage_fetch(moe_stager* s, const int32_t* ids, int32_t n, int32_t* n_enqueued);
 /* Whether module `id` currently occupies a slot (copied or copy in flight). */
 int moe_stage_resident(moe_stager* s, int32_t id);
-/* Grow (or shrink back) the number of usable slots of a type within the memory
- * given at creation: set_phase / resize_buffer / reset_prefill_buffer
- * (GPU_Weight_Buffer.cpp:103-142, 310-379).  reset != 0 also drops residency and
- * rewinds the cyclic queues (HtoD_Engine.cpp:284-311). */
+/* Low-level form of the phase verbs below: set the number of usable slots of a type within
+ * the memory given at creation.  reset != 0 also drops residency of the type and rewinds its
+ * cyclic queue; it fails with MOE_ERR_STATE while a module of the type is acquired and not
+ * released (its kernels may still be queued). */
 int moe_stage_set_active_slots(moe_stager* s, int32_t type, int32_t n_active, int32_t reset);
+
+/*
+ * The reference's remaining verbs on the pool (core/MoE_Gen_Binding.cpp:45-65).  Modules are
+ * named by tag instead of by string: moe_stage_tag_module(id, L, e) stands for the key
+ * "routed_expert_{L}_{e}" (e >= 0) or "shared_expert_{L}" (e == -1) of Wrapper.py:457-468.
+ */
+/* model_config.model_type ("deepseek_v2", "deepseek_v3", anything else), num_hidden_layers and
+ * num_local_experts, which clear_expert_buffer's previous-layer rule reads
+ * (GPU_Weight_Buffer.cpp:279-300). */
+int moe_stage_set_model(moe_stager* s, const char* model_type, int32_t num_hidden_layers,
+                        int32_t num_local_experts);
+int moe_stage_tag_module(moe_stager* s, int32_t id, int32_t layer_idx, int32_t expert_idx);
+/* clear_expert_buffer (GPU_Weight_Buffer::clear_expert_buffer, GPU_Weight_Buffer.cpp:261-308):
+ * release the slots of resident routed experts < expert_idx of layer_idx and of every routed
+ * expert of the previous layer -- experts that were prefetched and then skipped because no
+ * token was routed to them.  "Previous" is layer_idx - 1, except that layers 0-1 (deepseek_v2)
+ * or 0-3 (deepseek_v3) take the last layer.  The next copy into a released slot waits for
+ * `stream`.  Returns the number of modules released (>= 0) or a negative status. */
+int moe_stage_clear_expert_buffer(moe_stager* s, int32_t layer_idx, int32_t expert_idx, void* stream);
+/* Slots of a type in the prefill and in the decoding phase
+ * (GPU_Buffer_Config.num_prefill_module_buffer / num_decoding_module_buffer,
+ * deepseekv3_initializer.py:912-927); 1 <= n_prefill <= n_decoding <= slots given at creation.
+ * Takes effect at once for the current phase. */
+int moe_stage_set_phase_slots(moe_stager* s, int32_t type, int32_t n_prefill, int32_t n_decoding);
+/* set_phase (MoE_Gen::set_phase, core/MoE_Gen.cpp:128-134): "decoding" grows every pool to its
+ * decoding size (resize_buffer, GPU_Weight_Buffer.cpp:103-142); "prefill" only records the phase. */
+int moe_stage_set_phase(moe_stager* s, const char* phase);
+/* reset_prefill_buffer (GPU_Weight_Buffer.cpp:310-379): every pool back to its prefill size with
+ * all residency dropped.  Drains the copy stream (host wait); MOE_ERR_STATE while a module is
+ * acquired and not released. */
+int moe_stage_reset_prefill_buffer(moe_stager* s);
+/* reset_weight_copy_queue (HtoD_Engine.cpp:295-311): every cyclic queue back to registration order. */
+int moe_stage_reset_weight_copy_queue(moe_stager* s);
 /* Counters: copies issued, bytes issued. */
 int moe_stage_stats(moe_stager* s, int64_t* n_copies, int64_t* n_bytes);
 /* Host-blocking drain of the copy stream (teardown, tests). */

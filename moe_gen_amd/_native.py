@@ -33,7 +33,7 @@ SIGNATURES = {
                                   c_void_p, c_void_p, c_void_p]),
     "moe_dispatch_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32]),
     "moe_dispatch": (ctypes.c_int, [c_void_p, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p,
-                                    c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_size_t, c_void_p]),
+                                    c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_size_t, c_void_p]),
     "moe_grouped_workspace_bytes": (c_size_t, [c_int32, c_int32]),
     "moe_grouped_swiglu_bf16": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                                c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p,
@@ -75,6 +75,13 @@ SIGNATURES = {
     "moe_stage_release": (ctypes.c_int, [c_void_p, c_int32, c_void_p]),
     "moe_stage_resident": (ctypes.c_int, [c_void_p, c_int32]),
     "moe_stage_set_active_slots": (ctypes.c_int, [c_void_p, c_int32, c_int32, c_int32]),
+    "moe_stage_set_model": (ctypes.c_int, [c_void_p, ctypes.c_char_p, c_int32, c_int32]),
+    "moe_stage_tag_module": (ctypes.c_int, [c_void_p, c_int32, c_int32, c_int32]),
+    "moe_stage_clear_expert_buffer": (ctypes.c_int, [c_void_p, c_int32, c_int32, c_void_p]),
+    "moe_stage_set_phase_slots": (ctypes.c_int, [c_void_p, c_int32, c_int32, c_int32]),
+    "moe_stage_set_phase": (ctypes.c_int, [c_void_p, ctypes.c_char_p]),
+    "moe_stage_reset_prefill_buffer": (ctypes.c_int, [c_void_p]),
+    "moe_stage_reset_weight_copy_queue": (ctypes.c_int, [c_void_p]),
     "moe_stage_stats": (ctypes.c_int, [c_void_p, ctypes.POINTER(c_int64), ctypes.POINTER(c_int64)]),
     "moe_stage_sync": (ctypes.c_int, [c_void_p]),
     "moe_stage_destroy": (ctypes.c_int, [c_void_p]),

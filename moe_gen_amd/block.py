@@ -1,6 +1,7 @@
 """Shared machinery of the three MoE blocks: the SwiGLU MLP module, weight collection
 (resident parameters, fp8 + block scales, or an engine that hands weights out slot by
-slot) and the fused forward  router -> dispatch -> grouped SwiGLU -> combine."""
+slot, in waves when its pool is smaller than the layer) and the fused forward
+router -> dispatch -> grouped SwiGLU -> combine."""
 from __future__ import annotations
 
 import torch
@@ -108,7 +109,9 @@ class SwiGLUMLP(nn.Module):
         if not x2d.is_contiguous():
             x2d = x2d.contiguous()
         n = x2d.shape[0]
-        ptrs = collect_pointers([self], None)[0]
+        if engine_backed(self):
+            raise RuntimeError("SwiGLUMLP.forward: engine-backed weights are handled by the MoE block")
+        ptrs = collect_pointers([self], None)
         offsets = torch.tensor([0, n], dtype=torch.int32, device=x.device)
         return ops.grouped_swiglu(x2d, None, ptrs, offsets, n).view(*shape)
 
@@ -140,66 +143,119 @@ def _tensors_of(expert, fetched=None):
     return (*ws, *ss)
 
 
-def collect_pointers(experts, cache, counts=None):
-    """Pointer tables for a list of expert modules, plus the list of engine keys to release
-    once the kernels that read the weights are enqueued.
+def _pointer_table(rows):
+    """ExpertPointers from a list of (gate, up, down, s_gate, s_up, s_down) tuples."""
+    cols = list(zip(*rows))
+    fp8 = cols[0][0].dtype == FP8
+    return ops.expert_pointers(list(cols[0]), list(cols[1]), list(cols[2]),
+                               *((list(c) for c in cols[3:]) if fp8 else (None, None, None)))
 
-    counts: optional per-expert token counts (device int32 [E]).  When given and the engine can
-    stage on demand (it has `fetch`), only the experts with a non-zero count are copied, busiest
-    first, and the others get a placeholder pointer that no tile ever reads -- the reference
-    copies every expert of the layer blindly (HtoD_Engine.cpp:201-268).  Costs one host read of
-    E integers per call.
 
-    Experts backed by an engine (an Expert_Wrapper-like object with `core_engine`,
-    `get_weights=True` and `expert_weights_idx`) are fetched through
-    `core_engine.get_weights(key)` exactly as Wrapper.py:479-491 does; the caller frees them
-    with `free_weights_buffer(key)` (Wrapper.py:517).  Resident experts are cached in `cache`
-    (a dict) keyed on the storage addresses of the first and last expert."""
-    first = experts[0]
-    engine_backed = bool(getattr(first, "get_weights", False)) and hasattr(first, "core_engine")
-    if engine_backed:
-        cols = [[] for _ in range(6)]
-        keys = []
-        # every expert of the layer is fetched below, so none of this layer's slots can be left
-        # behind by a skipped expert; one call reclaims what the previous layer left
-        if getattr(first, "expert_idx", -1) != -1:
-            first.core_engine.clear_expert_buffer(first.layer_idx, 0)
-        hot = None
-        if counts is not None and hasattr(first.core_engine, "fetch"):
-            c_host = counts.tolist()
-            hot = sorted((e for e in range(len(experts)) if c_host[e] > 0), key=lambda e: -c_host[e])
-            first.core_engine.fetch([experts[e].expert_weights_idx for e in hot])
-        if hot is None:
-            chosen = range(len(experts))
-        else:
-            chosen = hot or [0]                  # no routed token at all: one expert stands in
-        got = {}
-        for e in chosen:
-            ex = experts[e]
-            fetched = ex.core_engine.get_weights(ex.expert_weights_idx)
-            keys.append((ex.core_engine, ex.expert_weights_idx))
-            got[e] = _tensors_of(ex, fetched)
-        stand_in = got[next(iter(chosen))]
-        for e in range(len(experts)):
-            for c, t in zip(cols, got.get(e, stand_in)):
-                c.append(t)
-        fp8 = cols[0][0].dtype == FP8
-        p = ops.expert_pointers(cols[0], cols[1], cols[2], *(cols[3:] if fp8 else (None, None, None)))
-        return p, keys
-    f = _tensors_of(first)
+def engine_backed(expert) -> bool:
+    """Whether an expert's weights come from an engine call by call: an Expert_Wrapper-like object
+    with `core_engine`, `get_weights=True` and `expert_weights_idx` (Wrapper.py:437-468)."""
+    return bool(getattr(expert, "get_weights", False)) and hasattr(expert, "core_engine")
+
+
+def collect_pointers(experts, cache):
+    """Pointer tables for a list of RESIDENT expert modules, cached in `cache` (a dict) keyed on
+    the storage addresses of the first and last expert."""
+    f = _tensors_of(experts[0])
     last = _tensors_of(experts[-1])
     stamp = (len(experts), f[0].data_ptr(), f[0].dtype, tuple(f[0].shape), last[2].data_ptr())
     if cache is not None and cache.get("stamp") == stamp:
-        return cache["ptrs"], []
-    cols = [[] for _ in range(6)]
-    for ex in experts:
-        for c, t in zip(cols, _tensors_of(ex)):
-            c.append(t)
-    fp8 = cols[0][0].dtype == FP8
-    p = ops.expert_pointers(cols[0], cols[1], cols[2], *(cols[3:] if fp8 else (None, None, None)))
+        return cache["ptrs"]
+    p = _pointer_table([_tensors_of(ex) for ex in experts])
     if cache is not None:
         cache["stamp"], cache["ptrs"] = stamp, p
-    return p, []
+    return p
+
+
+def pool_size(expert, module_type: str = "routed_expert") -> int:
+    """How many modules of `module_type` the engine behind `expert` can hold at once.
+
+    The library's Stager reports it (`pool_size`).  MoE-Gen's engine keeps it in the config the
+    wrapper carries: `engine_config.GPU_Buffer_Config.num_prefill_module_buffer[type]`, or
+    `num_decoding_module_buffer[type]` once `Expert_Wrapper.phase` is "decoding"
+    (deepseekv3_initializer.py:912-927, Wrapper.py:435).  Unknown: 1, the reference's own pattern
+    of one expert at a time (Wrapper.py:475-521)."""
+    eng = expert.core_engine
+    if callable(getattr(eng, "pool_size", None)):
+        return max(1, int(eng.pool_size(module_type)))
+    gb = getattr(getattr(expert, "engine_config", None), "GPU_Buffer_Config", None)
+    if gb is not None:
+        decoding = getattr(type(expert), "phase", "prefill") == "decoding"
+        table = gb.num_decoding_module_buffer if decoding else gb.num_prefill_module_buffer
+        if table and module_type in table:
+            return max(1, int(table[module_type]))
+    return 1
+
+
+def expert_waves(n_experts: int, pool: int, hot=None):
+    """Cut a layer's experts into waves that fit a pool of `pool` slots.
+
+    Returns a list of (first, last_plus_one, fetch_list): the grouped kernels of a wave run on the
+    experts [first, last_plus_one) and `fetch_list` names the ones whose weights the wave holds.
+    Without `hot` every expert is fetched, in id order, `pool` at a time -- the order in which the
+    reference's copy worker delivers them (HtoD_Engine.cpp:201-268), so a wave's weights are
+    exactly what the pool holds or receives next.  With `hot` (ids of the experts that received
+    tokens, on-demand staging) only those are fetched; a wave then spans from its first to its
+    last hot expert and the cold ones in between own no rows."""
+    pool = max(1, int(pool))
+    if hot is None:
+        return [(a, min(a + pool, n_experts), list(range(a, min(a + pool, n_experts)))) for a in range(0, n_experts, pool)]
+    hot = sorted(hot)
+    return [(hot[i], hot[min(i + pool, len(hot)) - 1] + 1, hot[i:i + pool]) for i in range(0, len(hot), pool)]
+
+
+def staged_experts_forward(experts, launch, counts_host=None, on_demand=False, stream_wait=None, module_type="routed_expert"):
+    """Run a layer's engine-backed experts through a pool that may be smaller than the layer.
+
+    Per wave (expert_waves): get_weights for the wave's experts, `launch(rows, first, last, n_rows)`
+    enqueues the grouped kernels for experts [first, last) with `rows[i]` the weight tensors of
+    expert first+i, then the wave's slots are released -- at once when the engine orders the
+    release on the stream itself (`stream_ordered_release`, the library's Stager), otherwise after
+    `stream_wait()` has drained the compute stream: the reference's pool marks a slot free on the
+    host and its copy thread overwrites it immediately (GPU_Weight_Buffer.cpp:163-169), which is
+    why Expert_Wrapper synchronises before free_weights_buffer (Wrapper.py:512-517).
+
+    counts_host: per-expert token counts on the host; needed when there is more than one wave (the
+    launch of a wave is sized by its own rows) and for on-demand staging.
+    on_demand: fetch only experts with tokens through the engine's `fetch` (busiest first when
+    they fit the pool at once)."""
+    first = experts[0]
+    eng = first.core_engine
+    E = len(experts)
+    pool = pool_size(first, module_type)
+    routed = getattr(first, "expert_idx", -1) != -1
+    if routed:
+        # every expert of the layer is fetched (or never copied, on demand), so none of this layer's
+        # slots is left behind by a skipped expert; one call reclaims what the previous layer left
+        eng.clear_expert_buffer(first.layer_idx, 0)
+    hot = None
+    if on_demand and counts_host is not None and hasattr(eng, "fetch"):
+        hot = [e for e in range(E) if counts_host[e] > 0]
+        if not hot:
+            return
+        if len(hot) <= pool:
+            hot_by_load = sorted(hot, key=lambda e: -counts_host[e])
+            eng.fetch([experts[e].expert_weights_idx for e in hot_by_load])
+    waves = expert_waves(E, pool, hot)
+    if len(waves) > 1 and counts_host is None:
+        raise RuntimeError("staged_experts_forward: more than one wave needs the per-expert counts on the host")
+    ordered = bool(getattr(eng, "stream_ordered_release", False))
+    for a, b, fetch in waves:
+        if hot is not None and len(hot) > pool:
+            eng.fetch([experts[e].expert_weights_idx for e in fetch])
+        got = {e: _tensors_of(experts[e], eng.get_weights(experts[e].expert_weights_idx)) for e in fetch}
+        stand_in = got[fetch[0]]                             # an expert without rows is never read
+        rows = [got.get(e, stand_in) for e in range(a, b)]
+        n_rows = None if counts_host is None else int(sum(counts_host[a:b]))
+        launch(rows, a, b, n_rows)
+        if not ordered and stream_wait is not None:
+            stream_wait()
+        for e in fetch:
+            eng.free_weights_buffer(experts[e].expert_weights_idx)
 
 
 def _gate_weight_bf16(weight: torch.Tensor, cache: dict) -> torch.Tensor:
@@ -215,6 +271,43 @@ def _gate_weight_bf16(weight: torch.Tensor, cache: dict) -> torch.Tensor:
             raise NotImplementedError("gate weight is not representable in bf16; the fused router reads bf16")
         cache["gate_key"], cache["gate_bf16"] = key, wb.contiguous()
     return cache["gate_bf16"]
+
+
+def _engine_experts(block, timer, tag, experts, a_rows, row_map, offsets, n_rows, counts):
+    """The expert MLPs of one layer with weights handed out by an engine, wave by wave."""
+    first = experts[0]
+    routed = tag == "routed"
+    mtype = "routed_expert" if routed else "shared_expert"
+    E = len(experts)
+    aware = routed and bool(getattr(block, "routing_aware_staging", False)) and hasattr(first.core_engine, "fetch")
+    counts_host = None
+    if routed and (aware or pool_size(first, mtype) < E):
+        counts_host = counts.tolist()                        # one read of E integers (the reference reads them too, :673)
+    hidden, inter = a_rows.shape[1], None
+    act = y = None
+
+    def launch(rows, a, b, rows_in_wave):
+        nonlocal act, y, inter
+        ptrs = _pointer_table(rows)
+        if y is None:
+            inter = ptrs.inter
+            act = torch.empty((n_rows, inter), dtype=torch.bfloat16, device=a_rows.device)
+            y = torch.empty((n_rows, hidden), dtype=torch.bfloat16, device=a_rows.device)
+        bound = n_rows if rows_in_wave is None else rows_in_wave
+        off = offsets[a:b + 1]
+        if timer is None:
+            ops.grouped_swiglu(a_rows, row_map, ptrs, off, n_rows, act, y, rows_bound=bound)
+        else:
+            with timer.span(tag + "_gate_up"):
+                ops.grouped_swiglu(a_rows, row_map, ptrs, off, n_rows, act, y, ops.PHASE_GATE_UP, rows_bound=bound)
+            with timer.span(tag + "_down"):
+                ops.grouped_swiglu(a_rows, row_map, ptrs, off, n_rows, act, y, ops.PHASE_DOWN, rows_bound=bound)
+
+    staged_experts_forward(experts, launch, counts_host, aware,
+                           stream_wait=lambda: torch.cuda.current_stream().synchronize(), module_type=mtype)
+    if y is None:                                            # no expert received a token
+        y = torch.empty((n_rows, hidden), dtype=torch.bfloat16, device=a_rows.device)
+    return y
 
 
 @torch.no_grad()
@@ -246,24 +339,26 @@ def moe_forward(block, hidden_states: torch.Tensor, spec: ops.RouterSpec, gate_w
     block.last_topk_idx, block.last_topk_weight = idx, w
     fused_gather = getattr(block, "fused_gather", True)
     with _span(timer, "dispatch"):
-        counts, offsets, perm, pos, xs = ops.dispatch(idx, E, None if fused_gather else x)
-        row_map = torch.div(perm, k, rounding_mode="floor").to(torch.int32) if fused_gather else None
+        d = ops.dispatch(idx, E, None if fused_gather else x, want_row_map=fused_gather)
+    counts, offsets, pos, row_map = d.counts, d.offsets, d.pos, d.row_map
     block.last_counts = counts
-    aware = counts if getattr(block, "routing_aware_staging", False) else None
-    ptrs, keys = collect_pointers(list(experts), cache.setdefault("routed", {}), aware)
-    y = _grouped(timer, "routed", x if fused_gather else xs, row_map, ptrs, offsets, n * k)
-    for eng, key in keys:
-        eng.free_weights_buffer(key)
+    experts = list(experts)
+    a_rows = x if fused_gather else d.xs
+    if engine_backed(experts[0]):
+        y = _engine_experts(block, timer, "routed", experts, a_rows, row_map, offsets, n * k, counts)
+    else:
+        y = _grouped(timer, "routed", a_rows, row_map, collect_pointers(experts, cache.setdefault("routed", {})),
+                     offsets, n * k)
     sh = None
     if shared is not None:
-        sp, skeys = collect_pointers([shared], cache.setdefault("shared", {}))
         so = cache.get("shared_off")
         if so is None or so[0] != n or so[1].device != x.device:
             so = (n, torch.tensor([0, n], dtype=torch.int32, device=x.device))
             cache["shared_off"] = so
-        sh = _grouped(timer, "shared", x, None, sp, so[1], n)
-        for eng, key in skeys:
-            eng.free_weights_buffer(key)
+        if engine_backed(shared):
+            sh = _engine_experts(block, timer, "shared", [shared], x, None, so[1], n, None)
+        else:
+            sh = _grouped(timer, "shared", x, None, collect_pointers([shared], cache.setdefault("shared", {})), so[1], n)
     with _span(timer, "combine"):
         out = ops.combine(y, pos, idx, w, sh, combine_mode, residual=residual)
     return out.view(*shape), logits

@@ -14,7 +14,8 @@
 //   2. scan_segments   : one wave per expert turns the per-segment counts into exclusive
 //                        bases across segments and writes counts[e]
 //   3. rank_scatter    : each block rebuilds offsets[] in LDS, ranks its entries with
-//                        wave-level match masks and writes perm / pos
+//                        wave-level match masks and writes perm / pos (and row_map = perm / k,
+//                        the token row behind each sorted row, for the GEMM's fused gather)
 // and one bandwidth kernel:
 //   4. gather_rows     : xs[r] = x[perm[r] / k], one wave per row, 16 bytes per lane.
 #include "common.h"
@@ -76,7 +77,7 @@ __global__ __launch_bounds__(256) void rank_scatter(const int32_t* __restrict__ 
                                                     const int32_t* __restrict__ seg_base,
                                                     const int32_t* __restrict__ counts,
                                                     int32_t* __restrict__ offsets, int32_t* __restrict__ perm,
-                                                    int32_t* __restrict__ pos) {
+                                                    int32_t* __restrict__ pos, int32_t* __restrict__ row_map, int k) {
     __shared__ int off[MAX_E];                 // exclusive prefix sum of counts
     __shared__ int whist[SEG_WAVES][MAX_E];    // per-wave counts, then per-wave running cursors
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -127,9 +128,12 @@ __global__ __launch_bounds__(256) void rank_scatter(const int32_t* __restrict__ 
     int* cur = whist[wave];
     for (int i0 = 0; i0 < SEG_PER_WAVE; i0 += 64) {
         int64_t g = wbase + i0 + lane;
-        bool ok = g < nk;
-        int e = ok ? idx[g] : 0;
-        ok = ok && (unsigned)e < (unsigned)E;
+        const bool in_list = g < nk;
+        int e = in_list ? idx[g] : 0;
+        const bool ok = in_list && (unsigned)e < (unsigned)E;
+        // an expert id outside [0, E) owns no sorted row: its slot points at row 0 so that a
+        // combine over this list reads valid memory
+        if (in_list && !ok) pos[g] = 0;
         uint64_t peers = __ballot(ok);
 #pragma unroll
         for (int b = 0; b < 8; ++b) {
@@ -142,6 +146,7 @@ __global__ __launch_bounds__(256) void rank_scatter(const int32_t* __restrict__ 
             int r = cur[e] + __popcll(below);
             perm[r] = (int32_t)g;
             pos[g] = r;
+            if (row_map) row_map[r] = (int32_t)(g / k);
         }
         // every read of cur[] above precedes this update in the wave's LDS order
         if (ok && (peers & ((1ull << lane) - 1ull)) == 0) cur[e] += __popcll(peers);
@@ -170,8 +175,9 @@ extern "C" size_t moe_dispatch_workspace_bytes(int32_t n_tokens, int32_t top_k, 
 }
 
 extern "C" int moe_dispatch(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k, int32_t n_experts,
-                            int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* pos, const void* x,
-                            int32_t hidden, void* xs, void* workspace, size_t workspace_bytes, void* stream) {
+                            int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* pos, int32_t* row_map,
+                            const void* x, int32_t hidden, void* xs, void* workspace, size_t workspace_bytes,
+                            void* stream) {
     using namespace moe;
     MOE_REQUIRE(n_tokens >= 0 && top_k >= 1, "moe_dispatch: bad n_tokens %d / top_k %d", n_tokens, top_k);
     MOE_REQUIRE(n_experts >= 1 && n_experts <= MAX_E, "moe_dispatch: n_experts %d outside [1,%d]", n_experts, MAX_E);
@@ -196,7 +202,7 @@ extern "C" int moe_dispatch(const int32_t* topk_idx, int32_t n_tokens, int32_t t
     hipLaunchKernelGGL(block_histogram, dim3(nseg), dim3(256), 0, st, topk_idx, nk, n_experts, seg);
     hipLaunchKernelGGL(scan_segments, dim3((n_experts + 3) / 4), dim3(256), 0, st, seg, nseg, n_experts, counts);
     hipLaunchKernelGGL(rank_scatter, dim3(nseg), dim3(256), 0, st, topk_idx, nk, n_experts, seg, counts, offsets, perm,
-                       pos);
+                       pos, row_map, top_k);
     if (x) {
         hipLaunchKernelGGL(gather_rows, dim3((unsigned)((nk + 3) / 4)), dim3(256), 0, st,
                            static_cast<const u32x4*>(x), perm, nk, top_k, hidden / 8, static_cast<u32x4*>(xs));

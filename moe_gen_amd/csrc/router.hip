@@ -72,13 +72,18 @@ __device__ __forceinline__ void butterfly(F&& step) {
     }
 }
 
+// Order of the selections: by value with NaN above every number (as torch.topk ranks it) and all
+// NaNs equal, so a NaN score is selected first, every lane of a group reaches the same decision and
+// the indices written stay inside [0, E); the NaN then travels on through the weights.
+__device__ __forceinline__ bool above(float a, float b) { return !(a <= b) && (b == b); }
+
 // max by value, equal values -> lower index
 template <int GW>
 __device__ __forceinline__ ArgMax group_argmax(ArgMax a) {
     butterfly<GW>([&](auto m) {
         const float ov = partner<decltype(m)::value>(a.v);
         const int oi = partner_bits<decltype(m)::value>(a.i);
-        const bool take = (ov > a.v) || (ov == a.v && oi < a.i);
+        const bool take = above(ov, a.v) || (!above(a.v, ov) && oi < a.i);
         a.v = take ? ov : a.v;
         a.i = take ? oi : a.i;
     });
@@ -161,7 +166,7 @@ __device__ void route_token(const float* row, const float* __restrict__ bias, co
             ArgMax a{kNegInf, kBigIdx};
 #pragma unroll
             for (int j = 0; j < MAX_EJ; ++j)
-                if (valid[j] && grp[j] == g && (c[j] > a.v || a.i == kBigIdx)) a = ArgMax{c[j], gl + GW * j};
+                if (valid[j] && grp[j] == g && (above(c[j], a.v) || a.i == kBigIdx)) a = ArgMax{c[j], gl + GW * j};
             a = group_argmax<GW>(a);
             float gs = a.v;
             if (p.method == MOE_TOPK_NOAUX_TC) {  // sum of the two largest of the group
@@ -197,7 +202,7 @@ __device__ void route_token(const float* row, const float* __restrict__ bias, co
         ArgMax a{kNegInf, kBigIdx};
 #pragma unroll
         for (int j = 0; j < MAX_EJ; ++j)
-            if (valid[j] && !taken[j] && (a.i == kBigIdx || tmp[j] > a.v)) a = ArgMax{tmp[j], gl + GW * j};
+            if (valid[j] && !taken[j] && (a.i == kBigIdx || above(tmp[j], a.v))) a = ArgMax{tmp[j], gl + GW * j};
         a = group_argmax<GW>(a);
         const int owner = a.i & (GW - 1), oj = a.i / GW;
         float sv = 0.0f;

@@ -18,6 +18,11 @@
 // the order they were registered, cyclically, whether or not the router will use them.
 // A type can instead be switched to on-demand: nothing is copied until the caller names the
 // modules it needs (fetch), typically the experts with a non-zero token count, busiest first.
+//
+// The reference's remaining verbs on the pool are here too, by module tag instead of by name:
+//   GPU_Weight_Buffer::clear_expert_buffer    GPU_Weight_Buffer.cpp:261-308  (moe_stage_clear_expert_buffer)
+//   MoE_Gen::set_phase -> resize_buffer       MoE_Gen.cpp:128-134            (moe_stage_set_phase)
+//   MoE_Gen::reset_prefill_buffer / reset_weight_copy_queue   MoE_Gen.cpp:205-211
 #include <cstring>
 #include <deque>
 #include <mutex>
@@ -36,6 +41,8 @@ struct Module {
     int type = 0;
     std::vector<Piece> pieces;
     int slot = -1;               // -1: not resident
+    bool held = false;           // acquired by a consumer and not yet released
+    int layer = -1, expert = -2; // tag: routed expert `expert` (>= 0) or shared expert (-1) of `layer`; -2 untagged
     hipEvent_t ready = nullptr;  // copy finished (device backend)
 };
 
@@ -49,6 +56,7 @@ struct Type {
     std::vector<int> order;             // registration order
     std::deque<int> fifo;               // cyclic copy queue
     int policy = MOE_STAGE_CYCLIC;
+    int n_prefill = 0, n_decoding = 0;  // slots per phase (0: the phase verbs leave this type alone)
 };
 
 }  // namespace
@@ -59,6 +67,9 @@ struct moe_stager {
     std::vector<Type> types;
     std::vector<Module> modules;
     int64_t n_copies = 0, n_bytes = 0;
+    int wrap_layers = 0;         // layers [0, wrap_layers) take the last layer as their "previous" one
+    int num_hidden_layers = 0, num_local_experts = 0;
+    int decoding = 0;
     std::mutex mu;
 };
 
@@ -99,8 +110,19 @@ int pump_type(moe_stager* st, int ti) {
     if (t.policy != MOE_STAGE_CYCLIC || t.fifo.empty()) return 0;
     const int slot = find_free(t);
     if (slot < 0) return 0;
+    // The next module in line that is not resident.  In the reference's order of use (modules
+    // released in the order they were copied) the head of the queue never is; if the caller let go
+    // of a later module first, resident ones keep their place in the cycle (they move to the back,
+    // as after a copy) instead of blocking the free slot -- the reference would copy the head a
+    // second time into the free slot (HtoD_Engine.cpp:201-268), which only costs bandwidth.
+    size_t turns = 0;
+    while (turns < t.fifo.size() && st->modules[t.fifo.front()].slot >= 0) {
+        t.fifo.push_back(t.fifo.front());
+        t.fifo.pop_front();
+        ++turns;
+    }
+    if (turns == t.fifo.size()) return 0;     // every module of the type is resident
     const int id = t.fifo.front();
-    if (st->modules[id].slot >= 0) return 0;  // next in line still occupies a slot: nothing to do until it is released
     t.fifo.pop_front();
     int rc = copy_into(st, id, slot);
     if (rc != MOE_OK) return rc;
@@ -121,6 +143,37 @@ int fetch_one(moe_stager* st, int id) {
     }
     int rc = copy_into(st, id, slot);
     return rc != MOE_OK ? rc : 1;
+}
+
+// hand the slot of a resident module back; the next copy into it waits for `stream`
+int release_one(moe_stager* st, int id, hipStream_t stream) {
+    Module& m = st->modules[id];
+    Type& t = st->types[m.type];
+    if (st->backend == MOE_STAGE_DEVICE) {
+        MOE_HIP_CHECK(hipEventRecord(t.freed[m.slot], stream));
+        t.freed_valid[m.slot] = 1;
+    }
+    t.owner[m.slot] = -1;
+    m.slot = -1;
+    m.held = false;
+    return MOE_OK;
+}
+
+// drop residency of every module of a type and rewind nothing: all its slots become free.  Refused
+// while a consumer holds one of them (its kernels may still be queued and no event covers them).
+int drop_residency(moe_stager* st, int ti, const char* who) {
+    Type& t = st->types[ti];
+    for (int s = 0; s < t.n_total; ++s)
+        if (t.owner[s] >= 0 && st->modules[t.owner[s]].held) {
+            moe::set_error("%s: module %d of type %d is still held (release it first)", who, t.owner[s], ti);
+            return MOE_ERR_STATE;
+        }
+    if (st->backend == MOE_STAGE_DEVICE) MOE_HIP_CHECK(hipStreamSynchronize(st->copy_stream));
+    for (int s = 0; s < t.n_total; ++s) {
+        if (t.owner[s] >= 0) st->modules[t.owner[s]].slot = -1;
+        t.owner[s] = -1;
+    }
+    return MOE_OK;
 }
 
 int pump_all(moe_stager* st) {
@@ -231,6 +284,7 @@ extern "C" int moe_stage_acquire(moe_stager* st, int32_t id, void* stream, int32
         }
     }
     if (st->backend == MOE_STAGE_DEVICE) MOE_HIP_CHECK(hipStreamWaitEvent(moe::as_stream(stream), m.ready, 0));
+    m.held = true;
     *slot = m.slot;
     return MOE_OK;
 }
@@ -244,15 +298,102 @@ extern "C" int moe_stage_release(moe_stager* st, int32_t id, void* stream) {
         moe::set_error("moe_stage_release: module %d is not resident", id);
         return MOE_ERR_STATE;
     }
-    Type& t = st->types[m.type];
-    if (st->backend == MOE_STAGE_DEVICE) {
-        MOE_HIP_CHECK(hipEventRecord(t.freed[m.slot], moe::as_stream(stream)));
-        t.freed_valid[m.slot] = 1;
-    }
-    t.owner[m.slot] = -1;
-    m.slot = -1;
+    int rc = release_one(st, id, moe::as_stream(stream));
+    if (rc != MOE_OK) return rc;
     int r = pump_all(st);  // the worker refills a freed slot at once
     return r < 0 ? r : MOE_OK;
+}
+
+extern "C" int moe_stage_set_model(moe_stager* st, const char* model_type, int32_t num_hidden_layers,
+                                   int32_t num_local_experts) {
+    MOE_REQUIRE(st && model_type, "moe_stage_set_model: NULL argument");
+    MOE_REQUIRE(num_hidden_layers >= 0 && num_local_experts >= 0, "moe_stage_set_model: negative count");
+    std::lock_guard<std::mutex> lk(st->mu);
+    // GPU_Weight_Buffer.cpp:279-294: the layers before the first MoE layer's successor wrap to the last layer
+    st->wrap_layers = std::strcmp(model_type, "deepseek_v2") == 0 ? 2 : std::strcmp(model_type, "deepseek_v3") == 0 ? 4 : 0;
+    st->num_hidden_layers = num_hidden_layers;
+    st->num_local_experts = num_local_experts;
+    return MOE_OK;
+}
+
+extern "C" int moe_stage_tag_module(moe_stager* st, int32_t id, int32_t layer_idx, int32_t expert_idx) {
+    MOE_REQUIRE(st, "moe_stage_tag_module: NULL stager");
+    std::lock_guard<std::mutex> lk(st->mu);
+    MOE_REQUIRE(id >= 0 && id < (int)st->modules.size(), "moe_stage_tag_module: unknown module id %d", id);
+    MOE_REQUIRE(layer_idx >= 0 && expert_idx >= -1, "moe_stage_tag_module: bad tag (layer %d, expert %d)", layer_idx,
+                expert_idx);
+    st->modules[id].layer = layer_idx;
+    st->modules[id].expert = expert_idx;
+    return MOE_OK;
+}
+
+extern "C" int moe_stage_clear_expert_buffer(moe_stager* st, int32_t layer_idx, int32_t expert_idx, void* stream) {
+    MOE_REQUIRE(st, "moe_stage_clear_expert_buffer: NULL stager");
+    std::lock_guard<std::mutex> lk(st->mu);
+    const int prev = (layer_idx >= 0 && layer_idx < st->wrap_layers) ? st->num_hidden_layers - 1 : layer_idx - 1;
+    int n = 0;
+    for (size_t id = 0; id < st->modules.size(); ++id) {
+        Module& m = st->modules[id];
+        if (m.slot < 0 || m.expert < 0) continue;                   // not resident / not a routed expert
+        const bool earlier = m.layer == layer_idx && m.expert < expert_idx;
+        const bool previous = m.layer == prev && m.expert < st->num_local_experts;
+        if (!earlier && !previous) continue;
+        int rc = release_one(st, (int)id, moe::as_stream(stream));
+        if (rc != MOE_OK) return rc;
+        ++n;
+    }
+    if (n > 0) {
+        int r = pump_all(st);
+        if (r < 0) return r;
+    }
+    return n;
+}
+
+extern "C" int moe_stage_set_phase_slots(moe_stager* st, int32_t type, int32_t n_prefill, int32_t n_decoding) {
+    MOE_REQUIRE(st, "moe_stage_set_phase_slots: NULL stager");
+    std::lock_guard<std::mutex> lk(st->mu);
+    MOE_REQUIRE(type >= 0 && type < (int)st->types.size(), "moe_stage_set_phase_slots: bad type %d", type);
+    Type& t = st->types[type];
+    MOE_REQUIRE(n_prefill >= 1 && n_prefill <= t.n_total && n_decoding >= n_prefill && n_decoding <= t.n_total,
+                "moe_stage_set_phase_slots: need 1 <= prefill %d <= decoding %d <= %d slots", n_prefill, n_decoding,
+                t.n_total);
+    for (int s = n_prefill; s < t.n_total; ++s)
+        MOE_REQUIRE(st->decoding || t.owner[s] < 0, "moe_stage_set_phase_slots: slot %d of type %d is occupied", s, type);
+    t.n_prefill = n_prefill;
+    t.n_decoding = n_decoding;
+    t.n_active = st->decoding ? n_decoding : n_prefill;
+    return MOE_OK;
+}
+
+extern "C" int moe_stage_set_phase(moe_stager* st, const char* phase) {
+    MOE_REQUIRE(st && phase, "moe_stage_set_phase: NULL argument");
+    std::lock_guard<std::mutex> lk(st->mu);
+    const bool dec = std::strcmp(phase, "decoding") == 0;
+    MOE_REQUIRE(dec || std::strcmp(phase, "prefill") == 0, "moe_stage_set_phase: unknown phase '%s'", phase);
+    st->decoding = dec ? 1 : 0;
+    if (dec)   // resize_buffer: the pools grow to their decoding size; nothing shrinks here
+        for (Type& t : st->types)
+            if (t.n_decoding > t.n_active) t.n_active = t.n_decoding;
+    return MOE_OK;
+}
+
+extern "C" int moe_stage_reset_prefill_buffer(moe_stager* st) {
+    MOE_REQUIRE(st, "moe_stage_reset_prefill_buffer: NULL stager");
+    std::lock_guard<std::mutex> lk(st->mu);
+    for (size_t ti = 0; ti < st->types.size(); ++ti) {
+        int rc = drop_residency(st, (int)ti, "moe_stage_reset_prefill_buffer");
+        if (rc != MOE_OK) return rc;
+    }
+    for (Type& t : st->types)
+        if (t.n_prefill > 0) t.n_active = t.n_prefill;
+    return MOE_OK;
+}
+
+extern "C" int moe_stage_reset_weight_copy_queue(moe_stager* st) {
+    MOE_REQUIRE(st, "moe_stage_reset_weight_copy_queue: NULL stager");
+    std::lock_guard<std::mutex> lk(st->mu);
+    for (Type& t : st->types) t.fifo.assign(t.order.begin(), t.order.end());
+    return MOE_OK;
 }
 
 extern "C" int moe_stage_set_policy(moe_stager* st, int32_t type, int32_t policy) {
@@ -298,11 +439,8 @@ extern "C" int moe_stage_set_active_slots(moe_stager* st, int32_t type, int32_t 
     MOE_REQUIRE(n_active >= 1 && n_active <= t.n_total, "moe_stage_set_active_slots: %d outside [1,%d]", n_active,
                 t.n_total);
     if (reset) {
-        if (st->backend == MOE_STAGE_DEVICE) MOE_HIP_CHECK(hipStreamSynchronize(st->copy_stream));
-        for (int s = 0; s < t.n_total; ++s) {
-            if (t.owner[s] >= 0) st->modules[t.owner[s]].slot = -1;
-            t.owner[s] = -1;
-        }
+        int rc = drop_residency(st, type, "moe_stage_set_active_slots");
+        if (rc != MOE_OK) return rc;
         t.fifo.assign(t.order.begin(), t.order.end());
     } else {
         for (int s = n_active; s < t.n_total; ++s)

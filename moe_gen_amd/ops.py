@@ -4,6 +4,7 @@ from __future__ import annotations
 
 import ctypes
 from dataclasses import dataclass
+from typing import NamedTuple
 
 import torch
 
@@ -77,9 +78,19 @@ def router(x: torch.Tensor, gate_w: torch.Tensor, bias, spec: RouterSpec, want_l
     return idx, w, lg
 
 
-def dispatch(topk_idx: torch.Tensor, n_experts: int, x: torch.Tensor | None = None):
-    """topk_idx int32 [n,k] -> counts [E], offsets [E+1], perm [n*k], pos [n*k] (int32) and,
-    if x bf16 [n,h] is given, the gathered rows xs [n*k,h]."""
+class Dispatch(NamedTuple):
+    counts: torch.Tensor             # int32 [E]
+    offsets: torch.Tensor            # int32 [E+1]
+    perm: torch.Tensor               # int32 [n*k]
+    pos: torch.Tensor                # int32 [n*k]
+    xs: torch.Tensor | None          # bf16 [n*k,h] gathered rows (only when x was given)
+    row_map: torch.Tensor | None     # int32 [n*k] = perm // k (only when asked for)
+
+
+def dispatch(topk_idx: torch.Tensor, n_experts: int, x: torch.Tensor | None = None, want_row_map: bool = False):
+    """topk_idx int32 [n,k] -> Dispatch(counts [E], offsets [E+1], perm [n*k], pos [n*k], xs, row_map):
+    if x bf16 [n,h] is given, xs holds the gathered rows [n*k,h]; with want_row_map, row_map[r] is
+    the token row behind sorted row r (the grouped GEMM gathers through it)."""
     _need(topk_idx, torch.int32, "topk_idx")
     n, k = topk_idx.shape
     dev = topk_idx.device
@@ -87,6 +98,7 @@ def dispatch(topk_idx: torch.Tensor, n_experts: int, x: torch.Tensor | None = No
     offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=dev)
     perm = torch.empty(n * k, dtype=torch.int32, device=dev)
     pos = torch.empty(n * k, dtype=torch.int32, device=dev)
+    row_map = torch.empty(n * k, dtype=torch.int32, device=dev) if want_row_map else None
     xs, h = None, 0
     if x is not None:
         _need(x, torch.bfloat16, "x")
@@ -97,8 +109,9 @@ def dispatch(topk_idx: torch.Tensor, n_experts: int, x: torch.Tensor | None = No
     wsb = N.lib().moe_dispatch_workspace_bytes(n, k, n_experts)
     ws = torch.empty(wsb, dtype=torch.uint8, device=dev)
     N.check(N.lib().moe_dispatch(_ptr(topk_idx), n, k, n_experts, _ptr(counts), _ptr(offsets), _ptr(perm),
-                                 _ptr(pos), _ptr(x), h, _ptr(xs), _ptr(ws), wsb, _stream()), "moe_dispatch")
-    return counts, offsets, perm, pos, xs
+                                 _ptr(pos), _ptr(row_map), _ptr(x), h, _ptr(xs), _ptr(ws), wsb, _stream()),
+            "moe_dispatch")
+    return Dispatch(counts, offsets, perm, pos, xs, row_map)
 
 
 @dataclass
@@ -152,9 +165,15 @@ PHASE_GATE_UP, PHASE_DOWN, PHASE_BOTH = 1, 2, 3
 
 
 def grouped_swiglu(x: torch.Tensor, row_map, ptrs: ExpertPointers, offsets: torch.Tensor, n_rows: int,
-                   act: torch.Tensor | None = None, y: torch.Tensor | None = None, phases: int = PHASE_BOTH):
+                   act: torch.Tensor | None = None, y: torch.Tensor | None = None, phases: int = PHASE_BOTH,
+                   rows_bound: int | None = None):
     """All experts' SwiGLU MLPs on their row ranges.  x: bf16 sorted rows [n_rows,h], or the
-    unsorted matrix with row_map int32 [n_rows].  Returns y bf16 [n_rows,h] (sorted-row order)."""
+    unsorted matrix with row_map int32 [n_rows].  Returns y bf16 [n_rows,h] (sorted-row order).
+
+    `ptrs` and `offsets` may describe a sub-range of a layer's experts (offsets = a slice
+    offsets[a:b+1] of the layer's, absolute sorted rows): x, row_map, act and y stay the layer's
+    full buffers, and rows_bound, if known, is the number of rows inside the range (it sizes the
+    launch and picks the tile shape; default: n_rows)."""
     _need(x, torch.bfloat16, "x")
     h, I, E = ptrs.hidden, ptrs.inter, ptrs.n_experts
     if x.shape[1] != h:
@@ -172,6 +191,10 @@ def grouped_swiglu(x: torch.Tensor, row_map, ptrs: ExpertPointers, offsets: torc
     _need(act, torch.bfloat16, "act", (n_rows, I))
     _need(y, torch.bfloat16, "y", (n_rows, h))
     L = N.lib()
+    if rows_bound is not None:
+        if not 0 <= rows_bound <= n_rows:
+            raise ValueError(f"rows_bound {rows_bound} outside [0, {n_rows}]")
+        n_rows = rows_bound
     if ptrs.fp8:
         N.check(L.moe_grouped_swiglu_w8a16(_ptr(x), _ptr(row_map), _ptr(ptrs.w_gate), _ptr(ptrs.w_up),
                                            _ptr(ptrs.w_down), _ptr(ptrs.s_gate), _ptr(ptrs.s_up),

@@ -1,17 +1,20 @@
-"""Expert-weight staging with the three verbs MoE-Gen's engine exposes to the model code
-(core/MoE_Gen_Binding.cpp:45-65): get_weights, free_weights_buffer, clear_expert_buffer, plus
-set_phase.  The slot pool and the copy queue live in libmoe_mi355.so (moe_stage_*); this class
-maps module keys ("routed_expert_{L}_{e}", "shared_expert_{L}", Wrapper.py:457-468) to ids and
-wraps slot memory as torch tensors."""
+"""Expert-weight staging with the verbs MoE-Gen's engine exposes to the model code
+(core/MoE_Gen_Binding.cpp:45-65): get_weights, free_weights_buffer, clear_expert_buffer,
+set_phase, reset_prefill_buffer, reset_weight_copy_queue.  The slot pool, the copy queue and all
+of these verbs live in libmoe_mi355.so (moe_stage_*); this class maps module keys
+("routed_expert_{L}_{e}", "shared_expert_{L}", Wrapper.py:457-468) to ids and tags and wraps slot
+memory as torch tensors."""
 from __future__ import annotations
 
 import ctypes
+import re
 
 import torch
 
 from . import _native as N
 
 _ALIGN = 256
+_KEY = re.compile(r"^(?:routed_expert_(\d+)_(\d+)|shared_expert_(\d+))$")
 
 
 def _nbytes(shape, dtype) -> int:
@@ -24,7 +27,7 @@ def _nbytes(shape, dtype) -> int:
 class StagedExpert(torch.nn.Module):
     """An expert whose weights live in pinned host memory and reach the GPU through a Stager (or
     MoE-Gen's core_engine): the attribute surface of the reference's Expert_Wrapper
-    (Wrapper.py:437-468) that block.collect_pointers consumes -- `.module`, `.core_engine`,
+    (Wrapper.py:437-468) that block.staged_experts_forward consumes -- `.module`, `.core_engine`,
     `.get_weights`, `.expert_weights_idx`, `.layer_idx`, `.expert_idx`, `.weight_dequant_scale`."""
 
     def __init__(self, expert_module, layer_idx: int, expert_idx: int, core_engine, weight_dequant_scale=None):
@@ -45,6 +48,11 @@ class Stager:
     counts for the decoding phase (num_decoding_module_buffer, :918-927);
     backend "device": slots in HBM, sources must be pinned host tensors;
     backend "host": slots in host memory, plain memcpy (host-only tests)."""
+
+    # free_weights_buffer records an event on the caller's stream and the next copy into the slot
+    # waits for it: a caller need not drain its stream before letting go of weights (the
+    # reference's pool flips a host flag, so its callers synchronise first, Wrapper.py:512-517)
+    stream_ordered_release = True
 
     def __init__(self, module_shapes: dict, n_slots: dict, device="cuda", n_slots_decoding: dict | None = None,
                  model_type: str = "", num_hidden_layers: int = 0, num_local_experts: int = 0,
@@ -77,10 +85,12 @@ class Stager:
         N.check(N.lib().moe_stage_create(ctypes.byref(self._h), nt, (ctypes.c_size_t * nt)(*slot_bytes),
                                          (ctypes.c_int32 * nt)(*totals), (ctypes.c_void_p * nt)(*mems),
                                          1 if backend == "host" else 0), "moe_stage_create")
+        N.check(N.lib().moe_stage_set_model(self._h, model_type.encode(), num_hidden_layers, num_local_experts),
+                "moe_stage_set_model")
         for i, t in enumerate(self.types):
-            if self.n_prefill[t] != totals[i]:
-                N.check(N.lib().moe_stage_set_active_slots(self._h, i, self.n_prefill[t], 0),
-                        "moe_stage_set_active_slots")
+            N.check(N.lib().moe_stage_set_phase_slots(self._h, i, self.n_prefill[t],
+                                                      max(self.n_prefill[t], self.n_decoding.get(t, 0))),
+                    "moe_stage_set_phase_slots")
         self.ids = {}          # module_key -> id
         self.type_of = {}      # module_key -> type
         self._src = []         # keeps the host tensors alive
@@ -109,9 +119,16 @@ class Stager:
                                            (ctypes.c_size_t * n)(*nbytes), (ctypes.c_size_t * n)(*offs))
         if mid < 0:
             N.check(mid, "moe_stage_add_module")
+        self._register(module_key, module_type, mid)
+        return mid
+
+    def _register(self, module_key: str, module_type: str, mid: int) -> None:
         self.ids[module_key] = mid
         self.type_of[module_key] = module_type
-        return mid
+        m = _KEY.match(module_key)
+        if m:        # the tag clear_expert_buffer selects by
+            layer, expert = (int(m.group(1)), int(m.group(2))) if m.group(1) is not None else (int(m.group(3)), -1)
+            N.check(N.lib().moe_stage_tag_module(self._h, mid, layer, expert), "moe_stage_tag_module")
 
     def add_module_from_arena(self, module_key: str, module_type: str, arena) -> int:
         """Register `module_key` with its tensors read in place from an Arena (the reference's
@@ -137,9 +154,12 @@ class Stager:
         if mid < 0:
             N.check(mid, "moe_stage_add_module_from_arena")
         self._src.append(arena)
-        self.ids[module_key] = mid
-        self.type_of[module_key] = module_type
+        self._register(module_key, module_type, mid)
         return mid
+
+    def pool_size(self, module_type: str) -> int:
+        """Slots of `module_type` usable in the current phase."""
+        return (self.n_decoding if self.phase == "decoding" else self.n_prefill)[module_type]
 
     def set_policy(self, module_type: str, policy: str) -> None:
         """"cyclic": every module of the type is copied in registration order whether or not it
@@ -192,39 +212,30 @@ class Stager:
             N.check(r, "moe_stage_resident")
         return bool(r)
 
-    def _prev_layer(self, layer_idx: int) -> int:
-        # GPU_Weight_Buffer.cpp:279-294: the first MoE layers wrap to the last layer
-        if self.model_type == "deepseek_v2" and layer_idx in (0, 1):
-            return self.num_hidden_layers - 1
-        if self.model_type == "deepseek_v3" and 0 <= layer_idx <= 3:
-            return self.num_hidden_layers - 1
-        return layer_idx - 1
-
-    def clear_expert_buffer(self, layer_idx: int, expert_idx: int) -> None:
+    def clear_expert_buffer(self, layer_idx: int, expert_idx: int) -> int:
         """Release slots still held by routed experts that were prefetched but skipped (no tokens):
         experts < expert_idx of this layer and every expert of the previous MoE layer
-        (GPU_Weight_Buffer::clear_expert_buffer, GPU_Weight_Buffer.cpp:261-308)."""
-        keys = [f"routed_expert_{layer_idx}_{e}" for e in range(expert_idx)]
-        pl = self._prev_layer(layer_idx)
-        keys += [f"routed_expert_{pl}_{e}" for e in range(self.num_local_experts)]
-        for key in keys:
-            if key in self.ids and self.resident(key):
-                self.free_weights_buffer(key)
+        (GPU_Weight_Buffer::clear_expert_buffer, GPU_Weight_Buffer.cpp:261-308).  Returns how many."""
+        r = N.lib().moe_stage_clear_expert_buffer(self._h, layer_idx, expert_idx, self._stream())
+        if r < 0:
+            N.check(r, "moe_stage_clear_expert_buffer")
+        return r
 
     def set_phase(self, phase: str) -> None:
-        """"decoding" grows the routed-expert pool (resize_buffer, GPU_Weight_Buffer.cpp:103-142);
-        "prefill" shrinks it back, drops residency and rewinds the queues
-        (reset_prefill_buffer :310-379, reset_weight_copy_queue HtoD_Engine.cpp:284-311)."""
-        if phase not in ("prefill", "decoding"):
-            raise RuntimeError(f"unknown phase {phase!r}")
-        for i, t in enumerate(self.types):
-            if phase == "decoding":
-                N.check(N.lib().moe_stage_set_active_slots(self._h, i, self.n_decoding.get(t, self.n_prefill[t]), 0),
-                        "moe_stage_set_active_slots")
-            else:
-                N.check(N.lib().moe_stage_set_active_slots(self._h, i, self.n_prefill[t], 1),
-                        "moe_stage_set_active_slots")
+        """"decoding" grows the pools to their decoding size (MoE_Gen::set_phase -> resize_buffer,
+        core/MoE_Gen.cpp:128-134, GPU_Weight_Buffer.cpp:103-142); "prefill" records the phase.  The
+        engine follows "prefill" with reset_prefill_buffer() and reset_weight_copy_queue()
+        (moe_gen/engine.py:680-683)."""
+        N.check(N.lib().moe_stage_set_phase(self._h, str(phase).encode()), "moe_stage_set_phase")
         self.phase = phase
+
+    def reset_prefill_buffer(self) -> None:
+        """Pools back to their prefill size, residency dropped (GPU_Weight_Buffer.cpp:310-379)."""
+        N.check(N.lib().moe_stage_reset_prefill_buffer(self._h), "moe_stage_reset_prefill_buffer")
+
+    def reset_weight_copy_queue(self) -> None:
+        """Cyclic queues back to registration order (HtoD_Engine.cpp:295-311)."""
+        N.check(N.lib().moe_stage_reset_weight_copy_queue(self._h), "moe_stage_reset_weight_copy_queue")
 
     def stats(self):
         c, b = ctypes.c_int64(), ctypes.c_int64()

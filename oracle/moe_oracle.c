@@ -194,12 +194,18 @@ static float canon_sum(const float* v, int n) {
     return p[0];
 }
 
+/* Order of every selection: by value, NaN above all numbers (the rank torch.topk gives it) and
+ * all NaNs equal.  The reference leaves NaN handling to the library; fixing this rule keeps the
+ * indices of a row with a NaN score well defined (inside [0, E), no duplicates) while the NaN
+ * itself travels on through the weights into the output, as it does in the reference. */
+static int above(float a, float b) { return !(a <= b) && (b == b); }
+
 /* argmax with "equal -> lower index"; entries with taken[e] != 0 are skipped */
 static int argmax_skip(const float* v, const uint8_t* taken, int n) {
     int best = -1;
     for (int e = 0; e < n; ++e) {
         if (taken[e]) continue;
-        if (best < 0 || v[e] > v[best]) best = e;
+        if (best < 0 || above(v[e], v[best])) best = e;
     }
     return best;
 }
@@ -256,7 +262,7 @@ static int route_one(const float* logit_in, const float* bias, const orc_router_
             const float* cg = c + g * per;
             if (p->method == 1) {                 /* max of the group */
                 float m = cg[0];
-                for (int i = 1; i < per; ++i) if (cg[i] > m) m = cg[i];
+                for (int i = 1; i < per; ++i) if (above(cg[i], m)) m = cg[i];
                 gs[g] = m;
             } else {                              /* sum of the two largest */
                 if (per < 2) return -3;

@@ -28,7 +28,7 @@ def test_dispatch_bit_exact(n, k, E, skew):
     idx = rand_idx(n, k, E, n + k + E, skew)
     h = 64
     x = torch.randn(n, h).to(torch.bfloat16)
-    counts, offsets, perm, pos, xs = ops.dispatch(torch.from_numpy(idx).cuda(), E, x.cuda())
+    counts, offsets, perm, pos, xs, row_map = ops.dispatch(torch.from_numpy(idx).cuda(), E, x.cuda(), want_row_map=True)
     torch.cuda.synchronize()
     oc, oo, op, opos = O.dispatch(idx, E)
     assert np.array_equal(counts.cpu().numpy(), oc)
@@ -36,16 +36,17 @@ def test_dispatch_bit_exact(n, k, E, skew):
     assert np.array_equal(perm.cpu().numpy(), op)
     assert np.array_equal(pos.cpu().numpy(), opos)
     assert np.array_equal(bits(xs), O.gather_rows(bits(x), op, k))
+    assert np.array_equal(row_map.cpu().numpy(), op // k)
 
 
 def test_dispatch_empty_and_unused_experts():
     from moe_gen_amd import ops
     idx = torch.zeros((0, 4), dtype=torch.int32, device="cuda")
-    counts, offsets, perm, pos, _ = ops.dispatch(idx, 16)
+    counts, offsets, perm, pos, _, _ = ops.dispatch(idx, 16)
     torch.cuda.synchronize()
     assert counts.sum().item() == 0 and offsets.sum().item() == 0 and perm.numel() == 0
     idx = torch.full((100, 1), 5, dtype=torch.int32, device="cuda")   # one expert takes everything
-    counts, offsets, perm, pos, _ = ops.dispatch(idx, 16)
+    counts, offsets, perm, pos, _, _ = ops.dispatch(idx, 16)
     assert counts.cpu().tolist() == [0] * 5 + [100] + [0] * 10
     assert perm.cpu().tolist() == list(range(100))
 
@@ -56,12 +57,34 @@ def test_dispatch_full_size_properties():
     n, k, E = 65536, 8, 256
     g = torch.Generator(device="cuda").manual_seed(3)
     idx = torch.rand((n, E), generator=g, device="cuda").topk(k, dim=1).indices.to(torch.int32)
-    counts, offsets, perm, pos, _ = ops.dispatch(idx, E)
+    counts, offsets, perm, pos, _, row_map = ops.dispatch(idx, E, want_row_map=True)
     flat = idx.view(-1).long()
     assert torch.equal(counts.long(), torch.bincount(flat, minlength=E))
     assert torch.equal(offsets[1:].long(), counts.long().cumsum(0)) and offsets[0].item() == 0
     assert torch.equal(perm.long(), torch.argsort(flat, stable=True))
     assert torch.equal(pos[perm.long()].long(), torch.arange(n * k, device="cuda"))
+    assert torch.equal(row_map, perm // k)
+
+
+def test_dispatch_ignores_out_of_range_ids():
+    """Ids outside [0, E) are not counted, own no sorted row and get pos 0, so a combine over the
+    list reads valid memory; the in-range entries are ranked as if the others were absent."""
+    from moe_gen_amd import ops
+    E, k = 16, 2
+    idx = rand_idx(200, k, E, 5)
+    bad = idx.copy()
+    bad[3, 1], bad[77, 0], bad[199, 1] = 0x7fffffff, -1, E
+    counts, offsets, perm, pos, _, _ = ops.dispatch(torch.from_numpy(bad).cuda(), E)
+    torch.cuda.synchronize()
+    flat = bad.reshape(-1)
+    good = (flat >= 0) & (flat < E)
+    assert np.array_equal(counts.cpu().numpy(), np.bincount(flat[good], minlength=E))
+    n_good = int(good.sum())
+    assert offsets.cpu().numpy()[-1] == n_good
+    order = np.flatnonzero(good)[np.argsort(flat[good], kind="stable")]
+    assert np.array_equal(perm.cpu().numpy()[:n_good], order)
+    p = pos.cpu().numpy()
+    assert np.array_equal(p[order], np.arange(n_good)) and (p[~good] == 0).all()
 
 
 @pytest.mark.parametrize("mode", [0, 1, 2])

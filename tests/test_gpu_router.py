@@ -116,7 +116,7 @@ def test_router_and_dispatch_golden_fixtures():
         bias = torch.from_numpy(z["bias"]) if "bias" in z.files else None
         idx, w, _ = gpu_router(bf16_tensor(z["x"]), bf16_tensor(z["gate"]), bias, spec)
         assert np.array_equal(idx, z["idx"]) and np.array_equal(w.view(np.uint32), z["w"].view(np.uint32)), f
-        counts, offsets, perm, pos, _ = ops.dispatch(torch.from_numpy(idx).cuda(), spec.n_experts)
+        counts, offsets, perm, pos, _, _ = ops.dispatch(torch.from_numpy(idx).cuda(), spec.n_experts)
         assert np.array_equal(counts.cpu().numpy(), z["counts"]) and np.array_equal(perm.cpu().numpy(), z["perm"])
         assert np.array_equal(offsets.cpu().numpy(), z["offsets"]) and np.array_equal(pos.cpu().numpy(), z["pos"])
 
@@ -197,3 +197,33 @@ def test_router_random_shapes_at_switch_points():
         assert np.array_equal(lg.view(np.uint32), ol.view(np.uint32)), (it, E, n, fam)
         assert np.array_equal(idx, oi), (it, E, n, fam)
         assert np.array_equal(w.view(np.uint32), ow.view(np.uint32)), (it, E, n, fam)
+
+
+@pytest.mark.parametrize("name", ["v3_256", "mixtral_8", "v2_group_160", "v2_greedy_64"])
+def test_router_nan_inputs_keep_indices_valid(name):
+    """NaN in a token row or in a gate row: selections rank NaN above every number (torch.topk's
+    order), so every lane group agrees, indices stay distinct and inside [0, E), and the NaN
+    travels into the weights -- identical to the oracle; dispatch and combine then run on valid
+    positions and the affected output rows are NaN."""
+    from moe_gen_amd import ops
+    spec, has_bias = FAMILIES[name]
+    n, h, E, k = 200, 256, spec.n_experts, spec.top_k
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(n, h, generator=g).to(torch.bfloat16)
+    wg = (torch.randn(E, h, generator=g) * 0.05).to(torch.bfloat16)
+    bias = (torch.randn(E, generator=g) * 0.01) if has_bias else None
+    x[3, 7] = float("nan"); x[150] = float("nan")          # whole rows of NaN logits
+    wg[min(5, E - 1), 100] = float("nan")                    # one expert's logit is NaN for every token
+    idx, w, _ = gpu_router(x, wg, bias, spec)
+    oi, ow, _ = O.router(bits(x), bits(wg), None if bias is None else bias.numpy(), spec)
+    assert idx.min() >= 0 and idx.max() < E and all(len(set(r)) == k for r in idx)
+    assert np.array_equal(idx, oi)
+    assert np.array_equal(np.isnan(w), np.isnan(ow))
+    ok = ~np.isnan(ow)
+    assert np.array_equal(w[ok].view(np.uint32), ow[ok].view(np.uint32))
+    d = ops.dispatch(torch.from_numpy(idx).cuda(), E)
+    y = torch.ones(n * k, 64, dtype=torch.bfloat16, device="cuda")
+    out = ops.combine(y, d.pos, torch.from_numpy(idx).cuda(), torch.from_numpy(w).cuda(), None,
+                      2 if name == "mixtral_8" else 0)
+    torch.cuda.synchronize()
+    assert np.array_equal(torch.isnan(out.float()).all(dim=1).cpu().numpy(), np.isnan(ow).any(axis=1))

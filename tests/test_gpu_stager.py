@@ -53,19 +53,71 @@ def test_stager_overlaps_with_compute():
     st.close()
 
 
-class FakeCoreEngine:
-    """Stands in for MoE-Gen's pybind `core_engine` (MoE_Gen_Binding.cpp:45-65): hands out device
-    tensors by module key and records the protocol calls."""
+def check_against_oracle(blk_resident, w, x_cpu, out, blk_run):
+    """Routing bit-exact and output within the layer bound (2e-2 of the fp32 oracle), as in
+    test_gpu_layer.py; `blk_resident` still owns the weights the oracle reads."""
+    import numpy as np
+    from oracle import oracle as O
+    from util import bits, oracle_spec, oracle_weights, rel_max
+    mode = {"v3": O.COMBINE_F32, "v2": O.COMBINE_BF16_PROD, "mixtral": O.COMBINE_BF16_SEQ}[w.family]
+    ref32, aux = O.layer(bits(x_cpu).reshape(w.n, w.h), oracle_weights(blk_resident, w.family), oracle_spec(w), mode,
+                         rounding="f32")
+    assert np.array_equal(blk_run.last_topk_idx.cpu().numpy(), aux["idx"])
+    assert np.array_equal(blk_run.last_counts.cpu().numpy(), aux["counts"])
+    err = rel_max(O.bf16_to_f32(bits(out)).reshape(w.n, w.h), ref32)
+    assert err <= 2e-2, err
 
-    def __init__(self, weights):
-        self.weights, self.calls, self.held = weights, [], set()
+
+class FakeCoreEngine:
+    """Stands in for MoE-Gen's pybind `core_engine` (MoE_Gen_Binding.cpp:45-65) with the reference's
+    slot semantics: a pool of `n_slots` device buffers per module type that a copy worker fills in
+    registration order whenever a slot is free (HtoD_Engine.cpp:201-268), a get_weights that can
+    only return what the worker delivered (GPU_Weight_Buffer.cpp:171-246; the reference spins, this
+    one raises), and a free_weights_buffer that lets the worker overwrite the slot AT ONCE
+    (GPU_Weight_Buffer.cpp:163-169) -- so a caller that frees while its kernels still read the slot
+    gets the next module's weights in its output."""
+
+    def __init__(self, weights, n_slots):
+        self.src = weights                                   # key -> {tensor name -> device tensor}
+        self.queue = {"routed_expert": [k for k in weights if k.startswith("routed")],
+                      "shared_expert": [k for k in weights if k.startswith("shared")]}
+        self.n_slots = dict(n_slots)
+        self.slots = {t: [None] * n for t, n in self.n_slots.items()}
+        self.mem = {t: [None] * n for t, n in self.n_slots.items()}
+        self.held, self.calls, self.max_held = set(), [], 0
+        self.side = torch.cuda.Stream()
+
+    @staticmethod
+    def _type(key):
+        return "routed_expert" if key.startswith("routed") else "shared_expert"
+
+    def _pump(self):
+        for t, q in self.queue.items():
+            while q and None in self.slots[t] and q[0] not in self.slots[t]:
+                s = self.slots[t].index(None)
+                key = q.pop(0); q.append(key)
+                if self.mem[t][s] is None:
+                    self.mem[t][s] = {n: torch.empty_like(v) for n, v in self.src[key].items()}
+                with torch.cuda.stream(self.side):          # the worker's own stream, then a host wait
+                    for n, v in self.src[key].items():
+                        self.mem[t][s][n].copy_(v)
+                self.side.synchronize()
+                self.slots[t][s] = key
 
     def get_weights(self, key):
-        self.calls.append(("get", key)); self.held.add(key)
-        return self.weights[key]
+        self._pump()
+        t = self._type(key)
+        if key not in self.slots[t]:
+            raise RuntimeError(f"get_weights({key}) would block forever: the pool holds {self.slots[t]}")
+        self.held.add(key); self.max_held = max(self.max_held, len(self.held))
+        self.calls.append(("get", key))
+        return self.mem[t][self.slots[t].index(key)]
 
     def free_weights_buffer(self, key):
         self.calls.append(("free", key)); self.held.remove(key)
+        t = self._type(key)
+        self.slots[t][self.slots[t].index(key)] = None
+        self._pump()                                         # the worker refills the slot immediately
 
     def clear_expert_buffer(self, layer_idx, expert_idx):
         self.calls.append(("clear", layer_idx, expert_idx))
@@ -73,24 +125,33 @@ class FakeCoreEngine:
 
 class ExpertWrapperLike(torch.nn.Module):
     """Attribute-for-attribute what the reference's Expert_Wrapper exposes (Wrapper.py:437-468)."""
+    phase = "prefill"
 
-    def __init__(self, module, layer_idx, expert_idx, core_engine, scales):
+    def __init__(self, module, layer_idx, expert_idx, core_engine, scales, engine_config):
         super().__init__()
         self.module, self.layer_idx, self.expert_idx = module, layer_idx, expert_idx
         self.core_engine, self.get_weights, self.weight_dequant_scale = core_engine, True, scales
+        self.engine_config = engine_config
         self.expert_weights_idx = (f"routed_expert_{layer_idx}_{expert_idx}" if expert_idx >= 0
                                    else f"shared_expert_{layer_idx}")
 
 
-@pytest.mark.parametrize("name", ["deepseek_v3_w8a16", "deepseek_v2_236b"])
-def test_block_with_engine_backed_experts(name):
-    """The block fed through MoE-Gen's expert-wrapper protocol gives the same bits as with resident
-    weights, and calls get_weights / free_weights_buffer once per expert."""
+@pytest.mark.parametrize("name,n_slots", [("deepseek_v3_w8a16", 20), ("deepseek_v2_236b", 20), ("deepseek_v3_w8a16", 256),
+                                          ("deepseek_v2_236b", 7)])
+def test_block_with_engine_backed_experts(name, n_slots):
+    """The block fed through MoE-Gen's expert-wrapper protocol against an engine with the
+    reference's default pool of 20 routed-expert slots (deepseekv3_initializer.py:912-916), far
+    fewer than the layer's experts: same bits as with resident weights, parity with the oracle,
+    never more than the pool held, one get/free per expert."""
+    from types import SimpleNamespace as NS
     from moe_gen_amd import synthetic
     w = synthetic.WORKLOADS[name].scaled(n=256, h=512, I=256, seq=64)
+    print(f"engine-backed {name} pool {n_slots} of {w.E} experts", flush=True)
     blk = synthetic.build_block(w, device="cuda", gen_device="cpu")
-    x = synthetic.hidden_states(w, "cpu").cuda()
+    x_cpu = synthetic.hidden_states(w, "cpu")
+    x = x_cpu.cuda()
     ref = blk(x).clone()
+    resident = synthetic.build_block(w, device="cuda", gen_device="cpu")     # keeps the weights for the oracle
     names = blk.experts[0].names
     L = 7
     weights, wrapped = {}, []
@@ -102,39 +163,53 @@ def test_block_with_engine_backed_experts(name):
             getattr(mlp, n).weight.data = torch.zeros(1, dtype=torch.bfloat16, device="cuda")
         return scales
 
-    eng = FakeCoreEngine(weights)
+    scales = [detach(ex, f"routed_expert_{L}_{e}") for e, ex in enumerate(blk.experts)]
+    sscale = detach(blk.shared_experts, f"shared_expert_{L}")
+    eng = FakeCoreEngine(weights, {"routed_expert": n_slots, "shared_expert": 1})
+    cfg = NS(GPU_Buffer_Config=NS(num_prefill_module_buffer={"routed_expert": n_slots, "shared_expert": 1},
+                                  num_decoding_module_buffer={"routed_expert": 4 * n_slots, "shared_expert": 1}))
     for e, ex in enumerate(blk.experts):
-        wrapped.append(ExpertWrapperLike(ex, L, e, eng, detach(ex, f"routed_expert_{L}_{e}")))
+        wrapped.append(ExpertWrapperLike(ex, L, e, eng, scales[e], cfg))
     blk.experts = torch.nn.ModuleList(wrapped)
-    blk.shared_experts = ExpertWrapperLike(blk.shared_experts, L, -1, eng, detach(blk.shared_experts, f"shared_expert_{L}"))
-    out = blk(x)
-    torch.cuda.synchronize()
-    assert torch.equal(out, ref)
+    blk.shared_experts = ExpertWrapperLike(blk.shared_experts, L, -1, eng, sscale, cfg)
+    for rep in range(2):                                  # the second call starts from a pool in mid-cycle
+        out = blk(x)
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref), rep
+    check_against_oracle(resident, w, x_cpu, out, blk)
+    assert eng.max_held <= max(n_slots, 1) and not eng.held
     gets = [c[1] for c in eng.calls if c[0] == "get"]
     frees = [c[1] for c in eng.calls if c[0] == "free"]
-    assert sorted(gets) == sorted(frees) == sorted(weights) and not eng.held
+    assert sorted(gets) == sorted(frees) == sorted(list(weights) * 2)
     assert ("clear", L, 0) in eng.calls
 
 
-def test_block_with_library_stager():
-    """Same, with the library's own Stager delivering fp8 experts from pinned host memory."""
+@pytest.mark.parametrize("routed_slots", [16, 5])
+def test_block_with_library_stager(routed_slots):
+    """Same, with the library's own Stager delivering fp8 experts from pinned host memory, with a
+    pool as large as the layer and with one smaller than it (waves)."""
     from moe_gen_amd import StagedExpert, Stager, synthetic
     w = synthetic.WORKLOADS["deepseek_v3_w8a16"].scaled(n=256, h=512, I=256, E=16, n_group=4, topk_group=2, k=4, seq=64)
     blk = synthetic.build_block(w, device="cuda", gen_device="cpu")
-    x = synthetic.hidden_states(w, "cpu").cuda()
+    resident = synthetic.build_block(w, device="cuda", gen_device="cpu")
+    x_cpu = synthetic.hidden_states(w, "cpu")
+    x = x_cpu.cuda()
     ref = blk(x).clone()
     names = blk.experts[0].names
     fp8 = torch.float8_e4m3fn
     shapes = {"routed_expert": {f"{n}.weight": (tuple(getattr(blk.experts[0], n).weight.shape), fp8) for n in names},
               "shared_expert": {f"{n}.weight": (tuple(getattr(blk.shared_experts, n).weight.shape), fp8) for n in names}}
-    st = Stager(shapes, {"routed_expert": w.E, "shared_expert": 1}, model_type="deepseek_v3", num_hidden_layers=8,
+    st = Stager(shapes, {"routed_expert": routed_slots, "shared_expert": 1}, model_type="deepseek_v3", num_hidden_layers=8,
                 num_local_experts=w.E)
     L = 5
     wrapped = []
     for e, ex in enumerate(blk.experts):
         st.add_module(f"routed_expert_{L}_{e}", "routed_expert",
                       {f"{n}.weight": getattr(ex, n).weight.data.cpu().pin_memory() for n in names})
-        wrapped.append(StagedExpert(ex, L, e, st, {f"{n}.weight_scale_inv": getattr(ex, n).weight_scale_inv.data for n in names}))
+        scales = {f"{n}.weight_scale_inv": getattr(ex, n).weight_scale_inv.data for n in names}
+        for n in names:                                    # the resident copy is gone: a stale pointer would show
+            getattr(ex, n).weight.data = torch.zeros(1, dtype=fp8, device="cuda")
+        wrapped.append(StagedExpert(ex, L, e, st, scales))
     sh = blk.shared_experts
     st.add_module(f"shared_expert_{L}", "shared_expert", {f"{n}.weight": getattr(sh, n).weight.data.cpu().pin_memory() for n in names})
     blk.experts = torch.nn.ModuleList(wrapped)
@@ -143,26 +218,31 @@ def test_block_with_library_stager():
         out = blk(x)
     torch.cuda.synchronize()
     assert torch.equal(out, ref)
+    check_against_oracle(resident, w, x_cpu, out, blk)
     assert st.stats()[0] >= 3 * (w.E + 1)
     st.close()
 
 
-def test_block_with_routing_aware_staging():
+@pytest.mark.parametrize("routed_slots", [64, 6])
+def test_block_with_routing_aware_staging(routed_slots):
     """With per-expert token counts on the host, only experts that received tokens are staged
-    (busiest first); the output is bit-identical to resident weights and the copy count equals the
-    number of such experts.  The reference's worker copies every expert of the layer."""
+    (busiest first when they fit the pool, else in waves); the output is bit-identical to resident
+    weights, in parity with the oracle, and the copy count equals the number of such experts.  The
+    reference's worker copies every expert of the layer."""
     from moe_gen_amd import StagedExpert, Stager, synthetic
     w = synthetic.WORKLOADS["deepseek_v3_w8a16"].scaled(n=24, h=512, I=256, E=64, n_group=8, topk_group=4, k=4, seq=8)
     blk = synthetic.build_block(w, device="cuda", gen_device="cpu")
-    x = synthetic.hidden_states(w, "cpu").cuda()
+    resident = synthetic.build_block(w, device="cuda", gen_device="cpu")
+    x_cpu = synthetic.hidden_states(w, "cpu")
+    x = x_cpu.cuda()
     ref = blk(x).clone()
     used = int((blk.last_counts > 0).sum())
-    assert 0 < used < w.E                                  # 24 tokens x 4 slots cannot reach all 64 experts
+    assert routed_slots < used < w.E or routed_slots == w.E    # 24 tokens x 4 slots cannot reach all 64 experts
     names = blk.experts[0].names
     fp8 = torch.float8_e4m3fn
     shapes = {"routed_expert": {f"{n}.weight": (tuple(getattr(blk.experts[0], n).weight.shape), fp8) for n in names},
               "shared_expert": {f"{n}.weight": (tuple(getattr(blk.shared_experts, n).weight.shape), fp8) for n in names}}
-    st = Stager(shapes, {"routed_expert": w.E, "shared_expert": 1}, model_type="deepseek_v3", num_hidden_layers=8,
+    st = Stager(shapes, {"routed_expert": routed_slots, "shared_expert": 1}, model_type="deepseek_v3", num_hidden_layers=8,
                 num_local_experts=w.E)
     st.set_policy("routed_expert", "on_demand")
     L = 5
@@ -187,6 +267,7 @@ def test_block_with_routing_aware_staging():
         assert torch.equal(out, ref), rep
         assert st.stats()[0] - c0 == used + 1, (rep, st.stats()[0] - c0, used)   # + the shared expert
         assert not any(st.resident(f"routed_expert_{L}_{e}") for e in range(w.E))
+    check_against_oracle(resident, w, x_cpu, out, blk)
     st.close()
 
 

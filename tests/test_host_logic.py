@@ -83,3 +83,130 @@ def test_zipf_bias_rides_on_feature_zero():
     b = g[:, 0].float()
     assert abs(b.mean().item()) < 0.02 and b.max() > 2.0 and b.min() < -0.5   # centred log-Zipf, skewed
     assert torch.equal(g, synthetic.gate_weight(w))                           # deterministic in the seed
+
+
+class _SlotLimitedEngine:
+    """A stand-in for MoE-Gen's core_engine whose pool has `n_slots` slots and whose copy worker
+    delivers modules in registration order (HtoD_Engine.cpp:201-268): get_weights of a module that
+    is not deliverable -- the pool is full of held modules, or modules in front of it in the queue
+    wait for a slot -- is the call on which the reference spins forever; here it raises."""
+
+    def __init__(self, keys, n_slots, on_demand=False):
+        self.queue, self.n_slots, self.on_demand = list(keys), n_slots, on_demand
+        self.resident, self.held, self.calls, self.synced = [], set(), [], True
+
+    def _pump(self):
+        while not self.on_demand and len(self.resident) < self.n_slots and self.queue[0] not in self.resident:
+            self.resident.append(self.queue[0])
+            self.queue.append(self.queue.pop(0))
+
+    def fetch(self, keys):
+        for key in keys:
+            if key not in self.resident:
+                assert len(self.resident) < self.n_slots, f"no free slot for {key}"
+                self.resident.append(key)
+
+    def get_weights(self, key):
+        self._pump()
+        assert key in self.resident, f"get_weights({key}) would block forever: pool holds {self.resident}"
+        self.held.add(key)
+        assert len(self.held) <= self.n_slots
+        self.calls.append(("get", key))
+        return {n + ".weight": torch.zeros(2, 2) for n in ("gate_proj", "up_proj", "down_proj")}
+
+    def free_weights_buffer(self, key):
+        assert self.synced, "slot released while kernels that read it may still run"
+        self.held.remove(key); self.resident.remove(key)
+        self.calls.append(("free", key))
+
+    def clear_expert_buffer(self, layer_idx, expert_idx):
+        self.calls.append(("clear", layer_idx, expert_idx))
+
+
+class _Wrapped(torch.nn.Module):
+    names = ("gate_proj", "up_proj", "down_proj")
+
+    def __init__(self, eng, L, e, engine_config=None):
+        super().__init__()
+        self.module = self
+        for n in self.names:
+            setattr(self, n, torch.nn.Linear(2, 2, bias=False))
+        self.layer_idx, self.expert_idx, self.core_engine, self.get_weights = L, e, eng, True
+        self.expert_weights_idx = f"routed_expert_{L}_{e}"
+        self.weight_dequant_scale = None
+        if engine_config is not None:
+            self.engine_config = engine_config
+
+
+def _engine_config(prefill, decoding):
+    from types import SimpleNamespace as NS
+    return NS(GPU_Buffer_Config=NS(num_prefill_module_buffer={"routed_expert": prefill, "shared_expert": 1},
+                                   num_decoding_module_buffer={"routed_expert": decoding, "shared_expert": 1}))
+
+
+@pytest.mark.parametrize("E,slots", [(64, 20), (8, 8), (8, 3), (5, 1), (256, 20)])
+def test_engine_pool_smaller_than_the_layer_runs_in_waves(E, slots):
+    """The reference's prefill pool holds 20 routed experts (deepseekv3_initializer.py:912-916) and
+    its get_weights blocks until the copy worker delivers (GPU_Weight_Buffer.cpp:171-246): the
+    block must never hold more than the pool, must ask for experts in delivery order, and must
+    drain the stream before it frees a slot of an engine that does not order releases itself."""
+    from moe_gen_amd import block
+    L = 5
+    keys = [f"routed_expert_{L}_{e}" for e in range(E)] + [f"routed_expert_{L + 1}_{e}" for e in range(E)]
+    eng = _SlotLimitedEngine(keys, slots)
+    experts = [_Wrapped(eng, L, e, _engine_config(slots, 4 * slots)) for e in range(E)]
+    assert block.pool_size(experts[0]) == slots
+    counts = [(7 * e) % 5 for e in range(E)]
+    launches = []
+
+    def launch(rows, a, b, n_rows):
+        assert len(rows) == b - a and all(f"routed_expert_{L}_{e}" in eng.held for e in range(a, b))
+        launches.append((a, b, n_rows))
+        eng.synced = False                                   # kernels reading the slots are now queued
+
+    def stream_wait():
+        eng.synced = True
+
+    block.staged_experts_forward(experts, launch, counts, stream_wait=stream_wait)
+    assert [a for a, _, _ in launches] == list(range(0, E, slots))
+    assert launches[-1][1] == E and all(b - a <= slots for a, b, _ in launches)
+    assert [n for _, _, n in launches] == [sum(counts[a:b]) for a, b, _ in launches]
+    assert not eng.held and eng.calls[0] == ("clear", L, 0)
+    gets = [c[1] for c in eng.calls if c[0] == "get"]
+    assert gets == keys[:E] and sorted(c[1] for c in eng.calls if c[0] == "free") == sorted(gets)
+    if E > slots:
+        with pytest.raises(RuntimeError, match="more than one wave"):
+            block.staged_experts_forward(experts, launch, None, stream_wait=stream_wait)
+
+
+def test_engine_phase_and_unknown_pool():
+    from moe_gen_amd import block
+    eng = _SlotLimitedEngine([f"routed_expert_0_{e}" for e in range(4)], 4)
+
+    class DecodingWrapped(_Wrapped):
+        phase = "decoding"
+
+    assert block.pool_size(DecodingWrapped(eng, 0, 0, _engine_config(2, 4))) == 4
+    assert block.pool_size(_Wrapped(eng, 0, 0, _engine_config(2, 4))) == 2
+    assert block.pool_size(_Wrapped(eng, 0, 0)) == 1          # nothing known: one at a time, as Wrapper.py:475-521
+    assert block.expert_waves(5, 2) == [(0, 2, [0, 1]), (2, 4, [2, 3]), (4, 5, [4])]
+    assert block.expert_waves(9, 2, hot=[7, 1, 4]) == [(1, 5, [1, 4]), (7, 8, [7])]
+
+
+def test_on_demand_waves_fetch_only_experts_with_tokens():
+    from moe_gen_amd import block
+    E, slots, L = 12, 3, 2
+    eng = _SlotLimitedEngine([f"routed_expert_{L}_{e}" for e in range(E)], slots, on_demand=True)
+    eng.pool_size = lambda module_type: slots
+    eng.stream_ordered_release = True
+    experts = [_Wrapped(eng, L, e) for e in range(E)]
+    counts = [0, 3, 0, 0, 9, 1, 0, 2, 0, 0, 5, 0]
+    launches = []
+    block.staged_experts_forward(experts, lambda rows, a, b, n: launches.append((a, b, n)), counts, on_demand=True)
+    assert launches == [(1, 6, 13), (7, 11, 7)]
+    assert [c[1] for c in eng.calls if c[0] == "get"] == [f"routed_expert_{L}_{e}" for e in (1, 4, 5, 7, 10)]
+    eng.calls.clear()
+    few = [0, 0, 4, 0, 0, 0, 0, 0, 6, 0, 0, 0]                # fits the pool: one wave, busiest first
+    launches.clear()
+    block.staged_experts_forward(experts, lambda rows, a, b, n: launches.append((a, b, n)), few, on_demand=True)
+    assert launches == [(2, 9, 10)] and not eng.held

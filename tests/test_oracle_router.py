@@ -219,3 +219,39 @@ def test_golden_fixtures():
         bias = z["bias"] if "bias" in z.files else None
         idx, w, lg = O.router(z["x"], z["gate"], bias, spec)
         assert np.array_equal(idx, z["idx"]) and np.array_equal(w.view(np.uint32), z["w"].view(np.uint32)), f
+
+
+def test_nan_scores_rank_above_every_number_as_in_torch_topk():
+    """The reference hands NaN scores to torch.topk, which ranks NaN above every number.  The
+    oracle's selections use that order (all NaNs equal, ties to the lower index), so the indices
+    of a row with NaN scores are distinct and in range and the NaN reaches the weights."""
+    rng = np.random.default_rng(11)
+    E, k, n = 32, 4, 64
+    lg = rng.normal(size=(n, E)).astype(np.float32)
+    nan_at = [rng.choice(E, size=1 + t % 3, replace=False) for t in range(n)]
+    for t, cols in enumerate(nan_at):
+        lg[t, cols] = np.nan
+    bias = (rng.normal(size=E) * 0.01).astype(np.float32)
+    spec = O.RouterSpec.deepseek_v3(E, k, 1, 1, True, 2.5)          # one group: plain top-k of sigmoid + bias
+    idx, w, sc = O.router_from_logits(lg, bias, spec, want_scores=True)
+    c = torch.from_numpy(sc) + torch.from_numpy(bias)
+    tidx = torch.topk(c, k, dim=-1).indices.numpy()
+    for t in range(n):
+        assert sorted(idx[t]) == sorted(tidx[t]), t                  # the library routine picks the same set
+        m = len(nan_at[t])
+        assert sorted(idx[t][:m]) == sorted(nan_at[t])               # NaNs first, in ascending index order
+        assert list(idx[t][:m]) == sorted(idx[t][:m])
+        assert np.isnan(w[t]).all()                                  # renormalised by a NaN sum
+    # group-limited: a group that holds a NaN has a NaN group score and is kept first
+    spec_g = O.RouterSpec.deepseek_v3(E, k, 4, 2, False, 1.0)
+    idx, w = O.router_from_logits(lg, bias, spec_g)
+    for t in range(n):
+        assert len(set(idx[t])) == k and idx[t].min() >= 0 and idx[t].max() < E
+        assert idx[t][0] == min(nan_at[t])
+        assert np.isnan(w[t][0])
+    # softmax: one NaN logit makes every score NaN; all equal -> the lowest indices in order
+    idx, w = O.router_from_logits(lg, None, O.RouterSpec.deepseek_v2(E, k))
+    assert (idx == np.arange(k)).all() and np.isnan(w).all()
+    for G, Kg in ((4, 2), (8, 3)):
+        idx, w = O.router_from_logits(lg, None, O.RouterSpec.deepseek_v2(E, k, "group_limited_greedy", G, Kg))
+        assert (idx == np.arange(k)).all() and np.isnan(w).all()

@@ -69,12 +69,89 @@ def test_fifo_reuse_and_clear_rule(model_type, first_moe):
     assert copies == len(model.copies)
 
 
-def test_prev_layer_wraps_for_first_moe_layers():
-    st, model, host, names = make("deepseek_v3", 6, 4, 4, 3)
-    assert st._prev_layer(3) == 5 and st._prev_layer(4) == 3 and model.prev_layer(3) == 5
-    st2 = Stager(SHAPES, {"routed_expert": 2, "shared_expert": 1}, backend="host", model_type="deepseek_v2",
-                 num_hidden_layers=27, num_local_experts=4)
-    assert st2._prev_layer(1) == 26 and st2._prev_layer(0) == 26 and st2._prev_layer(2) == 1
+@pytest.mark.parametrize("model_type,layers,wrapping", [("deepseek_v3", 6, (0, 1, 2, 3)), ("deepseek_v2", 27, (0, 1)),
+                                                        ("mixtral", 4, ())])
+def test_clear_rule_through_the_c_abi(model_type, layers, wrapping):
+    """moe_stage_clear_expert_buffer, driven by module tags through ctypes alone: experts below
+    expert_idx of the layer and every routed expert of the previous layer are released, the first
+    layers of the DeepSeek models take the last layer as previous (GPU_Weight_Buffer.cpp:279-294),
+    shared experts and other layers stay.  Checked against the Python slot-pool model."""
+    import ctypes
+    from moe_gen_amd import _native as N
+    L = N.lib()
+    E, nb = 3, 64
+    probe = sorted({0, 1, 2, 3, 4, layers - 1})               # layers that hold modules
+    n_mod = len(probe) * (E + 1)
+    pool = (ctypes.c_uint8 * (n_mod * nb))()
+    spool = (ctypes.c_uint8 * (len(probe) * nb))()
+    h = ctypes.c_void_p()
+    N.check(L.moe_stage_create(ctypes.byref(h), 2, (ctypes.c_size_t * 2)(nb, nb), (ctypes.c_int32 * 2)(len(probe) * E, len(probe)),
+                               (ctypes.c_void_p * 2)(ctypes.addressof(pool), ctypes.addressof(spool)), 1), "create")
+    N.check(L.moe_stage_set_model(h, model_type.encode(), layers, E), "set_model")
+    src = (ctypes.c_uint8 * nb)(*range(nb))
+    ids, names = {}, {"routed_expert": [], "shared_expert": []}
+    for lay in probe:
+        for e in list(range(E)) + [-1]:
+            mid = L.moe_stage_add_module(h, 0 if e >= 0 else 1, 1, (ctypes.c_void_p * 1)(ctypes.addressof(src)),
+                                         (ctypes.c_size_t * 1)(nb), (ctypes.c_size_t * 1)(0))
+            assert mid >= 0
+            N.check(L.moe_stage_tag_module(h, mid, lay, e), "tag")
+            key = f"routed_expert_{lay}_{e}" if e >= 0 else f"shared_expert_{lay}"
+            ids[key] = mid
+            names["routed_expert" if e >= 0 else "shared_expert"].append(key)
+    for lay in probe:
+        for upto in (0, 2):
+            # every module fits the pool: all resident before each clear, in the library and in a fresh model
+            model = SlotPoolModel({"routed_expert": len(probe) * E, "shared_expert": len(probe)}, names, model_type, layers, E)
+            for _ in range(n_mod):
+                model.pump()
+            assert L.moe_stage_pump(h) >= 0
+            assert all(L.moe_stage_resident(h, i) == 1 for i in ids.values()) and len(model.resident) == n_mod
+            before = set(model.resident)
+            model.clear_expert_buffer(lay, upto)
+            released = L.moe_stage_clear_expert_buffer(h, lay, upto, None)
+            assert released == len(before - set(model.resident))
+            prev = layers - 1 if lay in wrapping else lay - 1
+            want_gone = {f"routed_expert_{lay}_{e}" for e in range(upto)} | {f"routed_expert_{prev}_{e}" for e in range(E)}
+            assert before - set(model.resident) == want_gone & set(ids)
+            # the freed slots are refilled at once with the modules that are not resident
+            assert all(L.moe_stage_resident(h, i) == 1 for i in ids.values())
+    assert L.moe_stage_tag_module(h, 10 ** 6, 0, 0) == -1 and "unknown module" in N.last_error()
+    L.moe_stage_destroy(h)
+
+
+def test_release_out_of_order_does_not_block_the_queue():
+    """Five modules, four slots, the consumer lets go of a later module first: the freed slot takes
+    the next module in line that is not resident, and a later acquire of the released module finds
+    a slot.  (The reference's worker would copy the still-resident head a second time.)"""
+    st = Stager(SHAPES, {"routed_expert": 4, "shared_expert": 1}, backend="host", model_type="mixtral",
+                num_hidden_layers=1, num_local_experts=5)
+    for e in range(5):
+        st.add_module(f"routed_expert_0_{e}", "routed_expert",
+                      {n: torch.full(s, float(e)).to(d) for n, (s, d) in SHAPES["routed_expert"].items()})
+    for e in range(4):
+        st.get_weights(f"routed_expert_0_{e}")
+    st.free_weights_buffer("routed_expert_0_1")                # 4 takes the slot; queue head 0 is still held
+    assert st.resident("routed_expert_0_4") and not st.resident("routed_expert_0_1")
+    st.free_weights_buffer("routed_expert_0_2")                # heads 0 (held) and 4 (resident) keep their place: 1 is copied
+    assert st.resident("routed_expert_0_1")
+    w = st.get_weights("routed_expert_0_1")
+    assert float(w["gate_proj.weight"][0, 0]) == 1.0
+    assert st.stats()[0] == 6
+
+
+def test_reset_is_refused_while_a_module_is_held():
+    st = Stager(SHAPES, {"routed_expert": 2, "shared_expert": 1}, backend="host", model_type="mixtral",
+                num_hidden_layers=1, num_local_experts=3)
+    for e in range(3):
+        st.add_module(f"routed_expert_0_{e}", "routed_expert",
+                      {n: torch.full(s, float(e)).to(d) for n, (s, d) in SHAPES["routed_expert"].items()})
+    st.get_weights("routed_expert_0_0")
+    with pytest.raises(RuntimeError, match="still held"):
+        st.reset_prefill_buffer()
+    st.free_weights_buffer("routed_expert_0_0")
+    st.reset_prefill_buffer()
+    assert not any(st.resident(f"routed_expert_0_{e}") for e in range(3))
 
 
 def test_errors_and_phase_switch():
@@ -87,7 +164,8 @@ def test_errors_and_phase_switch():
     with pytest.raises(RuntimeError, match="not resident"):
         st.free_weights_buffer("routed_expert_1_3")
     st.free_weights_buffer("routed_expert_0_0"); st.free_weights_buffer("routed_expert_0_1")
-    # decoding phase may use more slots; prefill resets residency and rewinds the queue
+    # decoding phase may use more slots; back in prefill the engine resets residency and rewinds the
+    # queue (moe_gen/engine.py:680-683)
     big = Stager(SHAPES, {"routed_expert": 2, "shared_expert": 1}, n_slots_decoding={"routed_expert": 5, "shared_expert": 1},
                  backend="host", model_type="mixtral", num_hidden_layers=1, num_local_experts=6)
     for e in range(6):
@@ -96,8 +174,13 @@ def test_errors_and_phase_switch():
     assert big.pump() == 2
     big.set_phase("decoding")
     assert big.pump() == 3 and big.resident("routed_expert_0_4") and not big.resident("routed_expert_0_5")
+    assert big.pool_size("routed_expert") == 5
     big.set_phase("prefill")
-    assert not big.resident("routed_expert_0_0")
+    assert big.resident("routed_expert_0_0")               # set_phase("prefill") alone changes nothing
+    big.reset_prefill_buffer(); big.reset_weight_copy_queue()
+    assert not big.resident("routed_expert_0_0") and big.pool_size("routed_expert") == 2
+    with pytest.raises(RuntimeError, match="unknown phase"):
+        big.set_phase("warmup")
     assert big.pump() == 2 and big.resident("routed_expert_0_1") and not big.resident("routed_expert_0_2")
     with pytest.raises(RuntimeError):
         big.add_module("routed_expert_0_9", "routed_expert", {"gate_proj.weight": torch.zeros(1)})
