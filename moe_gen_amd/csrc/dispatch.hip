@@ -174,31 +174,14 @@ extern "C" size_t moe_dispatch_workspace_bytes(int32_t n_tokens, int32_t top_k, 
     return (size_t)(nseg * n_experts * 4 + 256);
 }
 
-extern "C" int moe_dispatch(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k, int32_t n_experts,
-                            int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* pos, int32_t* row_map,
-                            const void* x, int32_t hidden, void* xs, void* workspace, size_t workspace_bytes,
-                            void* stream) {
-    using namespace moe;
-    MOE_REQUIRE(n_tokens >= 0 && top_k >= 1, "moe_dispatch: bad n_tokens %d / top_k %d", n_tokens, top_k);
-    MOE_REQUIRE(n_experts >= 1 && n_experts <= MAX_E, "moe_dispatch: n_experts %d outside [1,%d]", n_experts, MAX_E);
-    MOE_REQUIRE(counts && offsets, "moe_dispatch: counts/offsets is NULL");
-    MOE_REQUIRE((x == nullptr) == (xs == nullptr), "moe_dispatch: x and xs must both be given or both be NULL");
-    const int64_t nk = (int64_t)n_tokens * top_k;
-    MOE_REQUIRE(nk < (int64_t)1 << 31, "moe_dispatch: n_tokens*top_k = %lld does not fit int32", (long long)nk);
-    hipStream_t st = as_stream(stream);
-    if (nk == 0) {
-        hipLaunchKernelGGL(zero_i32, dim3(2), dim3(256), 0, st, counts, n_experts, offsets, n_experts + 1);
-        MOE_HIP_CHECK(hipGetLastError());
-        return MOE_OK;
-    }
-    MOE_REQUIRE(topk_idx && perm && pos, "moe_dispatch: NULL index pointer");
-    if (x) MOE_REQUIRE(hidden > 0 && hidden % 8 == 0, "moe_dispatch: hidden %d must be a positive multiple of 8", hidden);
+namespace moe {
+namespace {
+
+// The launches behind both entry points; `seg` holds nseg * n_experts per-segment counts.
+int dispatch_launch(const int32_t* topk_idx, int64_t nk, int32_t top_k, int32_t n_experts, int32_t* counts,
+                    int32_t* offsets, int32_t* perm, int32_t* pos, int32_t* row_map, const void* x, int32_t hidden,
+                    void* xs, int32_t* seg, hipStream_t st) {
     const int nseg = (int)((nk + SEG - 1) / SEG);
-    if (workspace == nullptr || workspace_bytes < (size_t)nseg * n_experts * 4) {
-        set_error("moe_dispatch: workspace %zu bytes, need %zu", workspace_bytes, (size_t)nseg * n_experts * 4);
-        return MOE_ERR_WORKSPACE;
-    }
-    int32_t* seg = static_cast<int32_t*>(workspace);
     hipLaunchKernelGGL(block_histogram, dim3(nseg), dim3(256), 0, st, topk_idx, nk, n_experts, seg);
     hipLaunchKernelGGL(scan_segments, dim3((n_experts + 3) / 4), dim3(256), 0, st, seg, nseg, n_experts, counts);
     hipLaunchKernelGGL(rank_scatter, dim3(nseg), dim3(256), 0, st, topk_idx, nk, n_experts, seg, counts, offsets, perm,
@@ -209,4 +192,49 @@ extern "C" int moe_dispatch(const int32_t* topk_idx, int32_t n_tokens, int32_t t
     }
     MOE_HIP_CHECK(hipGetLastError());
     return MOE_OK;
+}
+
+// argument checks shared by the entry points; *nk_out = n_tokens * top_k
+int dispatch_check(const char* who, const int32_t* topk_idx, int32_t n_tokens, int32_t top_k, int32_t n_experts,
+                   int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* pos, const void* x, int32_t hidden,
+                   void* xs, int64_t* nk_out) {
+    MOE_REQUIRE(n_tokens >= 0 && top_k >= 1, "%s: bad n_tokens %d / top_k %d", who, n_tokens, top_k);
+    MOE_REQUIRE(n_experts >= 1 && n_experts <= MAX_E, "%s: n_experts %d outside [1,%d]", who, n_experts, MAX_E);
+    MOE_REQUIRE(counts && offsets, "%s: counts/offsets is NULL", who);
+    MOE_REQUIRE((x == nullptr) == (xs == nullptr), "%s: x and xs must both be given or both be NULL", who);
+    const int64_t nk = (int64_t)n_tokens * top_k;
+    MOE_REQUIRE(nk < (int64_t)1 << 31, "%s: n_tokens*top_k = %lld does not fit int32", who, (long long)nk);
+    if (nk > 0) {
+        MOE_REQUIRE(topk_idx && perm && pos, "%s: NULL index pointer", who);
+        if (x) MOE_REQUIRE(hidden > 0 && hidden % 8 == 0, "%s: hidden %d must be a positive multiple of 8", who, hidden);
+    }
+    *nk_out = nk;
+    return MOE_OK;
+}
+
+}  // namespace
+}  // namespace moe
+
+extern "C" int moe_dispatch(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k, int32_t n_experts,
+                            int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* pos, int32_t* row_map,
+                            const void* x, int32_t hidden, void* xs, void* workspace, size_t workspace_bytes,
+                            void* stream) {
+    using namespace moe;
+    int64_t nk = 0;
+    int rc = dispatch_check("moe_dispatch", topk_idx, n_tokens, top_k, n_experts, counts, offsets, perm, pos, x, hidden,
+                            xs, &nk);
+    if (rc != MOE_OK) return rc;
+    hipStream_t st = as_stream(stream);
+    if (nk == 0) {
+        hipLaunchKernelGGL(zero_i32, dim3(2), dim3(256), 0, st, counts, n_experts, offsets, n_experts + 1);
+        MOE_HIP_CHECK(hipGetLastError());
+        return MOE_OK;
+    }
+    const size_t need = (size_t)((nk + SEG - 1) / SEG) * n_experts * 4;
+    if (workspace == nullptr || workspace_bytes < need) {
+        set_error("moe_dispatch: workspace %zu bytes, need %zu", workspace_bytes, need);
+        return MOE_ERR_WORKSPACE;
+    }
+    return dispatch_launch(topk_idx, nk, top_k, n_experts, counts, offsets, perm, pos, row_map, x, hidden, xs,
+                           static_cast<int32_t*>(workspace), st);
 }
