@@ -107,6 +107,23 @@ int moe_dispatch(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k, int32
                  const void* x, int32_t hidden, void* xs,
                  void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * moe_dispatch without a workspace and without any allocation.  No counterpart in the reference:
+ * it exists for callers that cannot allocate device memory at the call -- code under HIP graph
+ * capture, tight serving loops, harnesses that forbid it.  The per-segment counters live in a
+ * device array built into the library (MOE_DISPATCH_STATIC_SCRATCH_BYTES on every GPU the
+ * library runs on, for the life of the process), which bounds the size of a call:
+ *     ceil(n_tokens * top_k / 2048) * n_experts * 4  <=  MOE_DISPATCH_STATIC_SCRATCH_BYTES
+ * (e.g. 2 097 152 routed entries with 256 experts, four times the DeepSeek-V3 workload at
+ * 65 536 tokens); larger calls fail with MOE_ERR_WORKSPACE and belong to moe_dispatch.  Same
+ * kernels, same results as moe_dispatch.  All calls on one GPU share the array: calls that
+ * overlap on one GPU (two streams, two threads) race; calls on one stream do not.
+ */
+#define MOE_DISPATCH_STATIC_SCRATCH_BYTES (1u << 20)
+int moe_dispatch_static(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k, int32_t n_experts,
+                        int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* pos, int32_t* row_map,
+                        const void* x, int32_t hidden, void* xs, void* stream);
+
 /* ----------------------------------------------------- grouped SwiGLU GEMM */
 
 /*

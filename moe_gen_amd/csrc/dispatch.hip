@@ -18,6 +18,8 @@
 //                        the token row behind each sorted row, for the GEMM's fused gather)
 // and one bandwidth kernel:
 //   4. gather_rows     : xs[r] = x[perm[r] / k], one wave per row, 16 bytes per lane.
+#include <mutex>
+
 #include "common.h"
 
 namespace moe {
@@ -237,4 +239,66 @@ extern "C" int moe_dispatch(const int32_t* topk_idx, int32_t n_tokens, int32_t t
     }
     return dispatch_launch(topk_idx, nk, top_k, n_experts, counts, offsets, perm, pos, row_map, x, hidden, xs,
                            static_cast<int32_t*>(workspace), st);
+}
+
+// ---- moe_dispatch_static: the same launches with the per-segment counts in a file-scope device
+// array instead of a caller workspace, for callers that cannot allocate.
+namespace moe {
+namespace {
+
+constexpr size_t STATIC_SCRATCH_INTS = MOE_DISPATCH_STATIC_SCRATCH_BYTES / sizeof(int32_t);
+// One copy per GPU the library runs on, held until the process ends.  block_histogram writes
+// every entry it later reads (all n_experts counts of all segments of the call), so a call needs
+// nothing cleared; what an earlier call left beyond that range is never read.
+static __device__ __align__(256) int32_t scratch[STATIC_SCRATCH_INTS];
+
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_mu;
+int32_t* scratch_ptr[MAX_DEVICES] = {nullptr};   // device address of `scratch` on each device
+
+// Device address of this GPU's copy of `scratch`, looked up once per device with that device
+// current.  (The array's name is only a host-side handle: kernels and copies take this pointer.)
+int static_scratch(int32_t** out) {
+    int dev = -1;
+    MOE_HIP_CHECK(hipGetDevice(&dev));
+    MOE_REQUIRE(dev >= 0 && dev < MAX_DEVICES, "moe_dispatch_static: device %d outside [0,%d)", dev, MAX_DEVICES);
+    std::lock_guard<std::mutex> lk(scratch_mu);
+    if (scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        MOE_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        MOE_REQUIRE(p != nullptr, "moe_dispatch_static: hipGetSymbolAddress returned NULL on device %d", dev);
+        scratch_ptr[dev] = static_cast<int32_t*>(p);
+    }
+    *out = scratch_ptr[dev];
+    return MOE_OK;
+}
+
+}  // namespace
+}  // namespace moe
+
+extern "C" int moe_dispatch_static(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k, int32_t n_experts,
+                                   int32_t* counts, int32_t* offsets, int32_t* perm, int32_t* pos, int32_t* row_map,
+                                   const void* x, int32_t hidden, void* xs, void* stream) {
+    using namespace moe;
+    int64_t nk = 0;
+    int rc = dispatch_check("moe_dispatch_static", topk_idx, n_tokens, top_k, n_experts, counts, offsets, perm, pos, x,
+                            hidden, xs, &nk);
+    if (rc != MOE_OK) return rc;
+    const size_t need = (size_t)((nk + SEG - 1) / SEG) * n_experts;
+    if (need > STATIC_SCRATCH_INTS) {
+        set_error("moe_dispatch_static: ceil(n_tokens*top_k / %d) * n_experts = %zu counters exceed the built-in "
+                  "scratch of %zu (%zu bytes); use moe_dispatch with a workspace", SEG, need, STATIC_SCRATCH_INTS,
+                  (size_t)MOE_DISPATCH_STATIC_SCRATCH_BYTES);
+        return MOE_ERR_WORKSPACE;
+    }
+    hipStream_t st = as_stream(stream);
+    if (nk == 0) {
+        hipLaunchKernelGGL(zero_i32, dim3(2), dim3(256), 0, st, counts, n_experts, offsets, n_experts + 1);
+        MOE_HIP_CHECK(hipGetLastError());
+        return MOE_OK;
+    }
+    int32_t* seg = nullptr;
+    rc = static_scratch(&seg);
+    if (rc != MOE_OK) return rc;
+    return dispatch_launch(topk_idx, nk, top_k, n_experts, counts, offsets, perm, pos, row_map, x, hidden, xs, seg, st);
 }
