@@ -1,11 +1,13 @@
 """MoE-layer benchmark on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--headline-only] [--no-cpu-baseline]
 
 A step is one forward of the MoE block (router -> dispatch -> grouped SwiGLU experts -> shared
 expert -> combine) over one batch of synthetic hidden states already resident in HBM, weights
-resident.  Prints ONE JSON line.  Per-stage durations come from events recorded on the launch
-stream inside the timed steps.
+resident.  Prints ONE JSON line: the DeepSeek-V3 W8A16 workload the metric is quoted on, with the
+same figures (tokens/s, roofline of the dominant kernel, routing GB/s, CPU baseline) for every
+other synthetic workload under "workloads".  Per-stage durations come from events recorded on the
+launch stream inside the timed steps.
 """
 import argparse
 import json
@@ -22,10 +24,23 @@ PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_HBM_GBPS = 8000.0
 
 
-def cpu_baseline(w, blk, n_sample: int):
+def cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    import platform
+    return platform.processor() or platform.machine()
+
+
+def cpu_baseline(w, blk, n_sample: int, passes: int = 3):
     """The reference's own algorithm (oracle/torch_blocks.py: fp32 gate, Python loop over experts,
     bf16 F.linear, per-call fp8 block dequantisation) timed on the host cores on a bounded sample
-    of the same workload: the first n_sample tokens, same weights, same router."""
+    of the same workload: the first n_sample tokens, same weights, same router.  One warm-up pass,
+    then the median of `passes` timed passes."""
     import torch
     from moe_gen_amd import synthetic
     from oracle import torch_blocks as TB
@@ -53,12 +68,17 @@ def cpu_baseline(w, blk, n_sample: int):
         return TB.deepseek_block(x, gate_w, bias, experts, shared, w.family, w.k, w.method, w.n_group,
                                  w.topk_group, w.norm, w.scale)
 
-    t0 = time.perf_counter()
-    run()
-    dt = time.perf_counter() - t0
-    return {"value": n_sample / dt, "unit": "tokens/s", "cores": threads, "kind": "port",
-            "sample": f"first {n_sample} of {w.n} tokens of the same workload, all experts' weights, one pass "
-                      f"({dt:.1f} s); stock-PyTorch CPU restatement of the reference block"}
+    run()                                            # warm-up: thread pool, allocator, page faults
+    times = []
+    for _ in range(passes):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    dt = sorted(times)[len(times) // 2]
+    return {"value": n_sample / dt, "unit": "tokens/s", "cores": threads, "cpu": cpu_model(), "kind": "port",
+            "sample": f"first {n_sample} of {w.n} tokens of the same workload, all experts' weights; one warm-up pass, "
+                      f"median of {passes} timed passes ({dt:.2f} s; all: {', '.join(f'{t:.2f}' for t in times)}); "
+                      "stock-PyTorch CPU restatement of the reference block"}
 
 
 def staged_run(w, blk, x, steps: int, routing_aware: bool = False):
@@ -173,26 +193,39 @@ def decoder_half_run(w, blk, x, steps: int):
             fn()
         torch.cuda.synchronize()
         out[name + "_ms_per_step"] = (_t.perf_counter() - t0) * 1e3 / steps
-    timer = StageTimer()
-    blk.stage_timer = timer
+    def stage_means(fn):
+        timer = StageTimer()
+        blk.stage_timer = timer
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        blk.stage_timer = None
+        return {k: sum(v) / len(v) for k, v in timer.totals_ms().items()}
+
+    st_f, st_p = stage_means(fused), stage_means(lambda: blk(x))
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    xf = x.view(-1, w.h)
+    a.record()
     for _ in range(steps):
-        fused()
+        ops.rmsnorm(xf, ln, 1e-6)
+    b.record()
     torch.cuda.synchronize()
-    blk.stage_timer = None
-    st = {k: sum(v) / len(v) for k, v in timer.totals_ms().items()}
     nh2 = 2.0 * w.n * w.h
-    out["rmsnorm_ms"] = st["rmsnorm"]
-    out["rmsnorm_gbps"] = 2 * nh2 / (st["rmsnorm"] * 1e-3) / 1e9            # read x, write the normalised copy
-    out["combine_residual_ms"] = st["combine"]
-    out["combine_residual_gbps"] = (w.combine_bytes + nh2) / (st["combine"] * 1e-3) / 1e9
+    out["rmsnorm_kernel_ms"] = a.elapsed_time(b) / steps
+    out["rmsnorm_kernel_gbps"] = 2 * nh2 / (out["rmsnorm_kernel_ms"] * 1e-3) / 1e9     # read x, write the normalised copy
+    out["router_ms"] = st_p["router"]
+    out["router_through_norm_ms"] = st_f["router"]        # norm folded into the router's read of the rows
+    out["combine_ms"] = st_p["combine"]
+    out["combine_residual_ms"] = st_f["combine"]
+    out["combine_residual_gbps"] = (w.combine_bytes + nh2) / (st_f["combine"] * 1e-3) / 1e9
     return out
 
 
 # HBM traffic per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (two runs; FETCH_SIZE scaled by 2.0, the factor a plain copy kernel of known size showed on this
-# box, WRITE_SIZE by 1.0).  bench.py cannot run the profiler on itself, so the figures are recorded
-# here from profiles/ for the workloads that were profiled; None elsewhere.
-MEASURED_TRAFFIC_BYTES = {"deepseek_v3_w8a16": 21.6e9}   # profiles/pmc_traffic_deepseek_v3_w8a16_65536.md
+# box, WRITE_SIZE by 1.0).  bench.py cannot run the profiler on itself: these are RECORDED figures,
+# copied from the named summary under profiles/, for the workloads that were profiled; None elsewhere.
+MEASURED_TRAFFIC = {"deepseek_v3_w8a16": (21.6e9, "profiles/pmc_traffic_deepseek_v3_w8a16_65536.md")}
 
 
 def run_workload(name: str, args, with_cpu: bool):
@@ -257,7 +290,9 @@ def run_workload(name: str, args, with_cpu: bool):
                                 if mt == 4 and w.E <= 512 and w.h % 128 == 0 else
                                 f"grouped_gemm_kernel<MT={mt},WN=4,SWIGLU=true,W8={'true' if w.fp8 else 'false'}> (gate/up + SiLU*mul)"),
                      "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(name),
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC.get(name, (None, None))[0],
+                     "traffic_source": (f"recorded from {MEASURED_TRAFFIC[name][1]} (rocprofv3 --pmc), not measured by this run"
+                                        if name in MEASURED_TRAFFIC else None),
                      "frac_of_fp8_peak": achieved / PEAK_FP8_TFLOPS,
                      "launches_per_step": len(gu_ms), "avg_launch_ms": ms_per_launch,
                      "flop_per_launch": flop_per_launch},
@@ -283,13 +318,102 @@ def run_workload(name: str, args, with_cpu: bool):
     return result
 
 
+def ceiling_run(args):
+    """What this box leaves to ANY bf16 GEMM of the headline shapes, next to the grouped kernel's own
+    dense (one-group) launch: (1) the registers-only MFMA loop of moe_gen_amd/csrc/probes/mfma_rate.hip,
+    (2) the vendor library's dense bf16 GEMM (torch.matmul) and (3) the library's grouped SwiGLU
+    kernels on one group of the same shape -- each with random and with all-zero operands.  The gap
+    between zero and random operands is data-dependent power, paid in clock."""
+    import subprocess
+
+    probe = os.path.join(ROOT, "moe_gen_amd", "csrc", "build", "mfma_rate")
+    if not os.path.exists(probe):
+        sys.exit(f"{probe} is missing: build it with make -C moe_gen_amd/csrc")
+    res = {"metric": "bf16 MFMA ceiling probes (DeepSeek-V3 MoE shapes)", "unit": "TFLOP/s", "peak": PEAK_BF16_TFLOPS}
+    # (1) started as a child before this process touches the GPU
+    txt = subprocess.run([probe, "10000"], check=True, capture_output=True, text=True, timeout=300).stdout
+    regs = {}
+    for line in txt.splitlines():
+        f = line.split()
+        if len(f) == 6 and f[0].startswith("mfma_"):
+            regs.setdefault(f"{f[0]}/{f[1]}", []).append(float(f[4]))
+    res["registers_only_mfma"] = {k: max(v) for k, v in regs.items()}
+
+    import torch
+    from moe_gen_amd import ops
+    torch.cuda.set_device(0)
+    dev = "cuda:0"
+    n, h, inter = 65536, 7168, 2048
+    reps = args.steps
+
+    def timed(fn):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / reps
+
+    g = torch.Generator(device=dev).manual_seed(0)
+
+    def tensor(shape, scale, zero):
+        if zero:
+            return torch.zeros(shape, dtype=torch.bfloat16, device=dev)
+        return (torch.randn(shape, generator=g, device=dev) * scale).to(torch.bfloat16)
+
+    vendor, ours = {}, {}
+    for zero in (False, True):
+        tag = "zero" if zero else "random"
+        x = tensor((n, h), 1.0, zero)
+        w_gu = tensor((2 * inter, h), 0.02, zero)             # gate and up as one dense matrix
+        w_d = tensor((h, inter), 0.02, zero)
+        act = tensor((n, inter), 0.05, zero)
+        c1 = torch.empty((n, 2 * inter), dtype=torch.bfloat16, device=dev)
+        c2 = torch.empty((n, h), dtype=torch.bfloat16, device=dev)
+        ms = timed(lambda: torch.matmul(x, w_gu.t(), out=c1))
+        vendor[f"gate_up_{n}x{2 * inter}x{h}/{tag}"] = 2.0 * n * 2 * inter * h / ms / 1e9
+        ms = timed(lambda: torch.matmul(act, w_d.t(), out=c2))
+        vendor[f"down_{n}x{h}x{inter}/{tag}"] = 2.0 * n * h * inter / ms / 1e9
+        del c1
+        ptrs = ops.expert_pointers([w_gu[:inter]], [w_gu[inter:]], [w_d])
+        off = torch.tensor([0, n], dtype=torch.int32, device=dev)
+        a2 = torch.empty((n, inter), dtype=torch.bfloat16, device=dev)
+        ms = timed(lambda: ops.grouped_swiglu(x, None, ptrs, off, n, a2, c2, ops.PHASE_GATE_UP))
+        ours[f"gate_up_swiglu_bf16/{tag}"] = 4.0 * n * inter * h / ms / 1e9
+        a2.copy_(act)
+        ms = timed(lambda: ops.grouped_swiglu(x, None, ptrs, off, n, a2, c2, ops.PHASE_DOWN))
+        ours[f"down_bf16/{tag}"] = 2.0 * n * h * inter / ms / 1e9
+        if not zero:                                          # the W8A16 path on the same shape
+            q = [torch.randint(0, 120, s, generator=g, device=dev, dtype=torch.uint8).view(torch.float8_e4m3fn)
+                 for s in ((inter, h), (inter, h), (h, inter))]
+            sc = [torch.full((-(-s[0] // 128), -(-s[1] // 128)), 1e-3, device=dev) for s in ((inter, h), (inter, h), (h, inter))]
+            p8 = ops.expert_pointers([q[0]], [q[1]], [q[2]], [sc[0]], [sc[1]], [sc[2]])
+            ms = timed(lambda: ops.grouped_swiglu(x, None, p8, off, n, a2, c2, ops.PHASE_GATE_UP))
+            ours["gate_up_swiglu_w8a16/random"] = 4.0 * n * inter * h / ms / 1e9
+            a2.copy_(act)
+            ms = timed(lambda: ops.grouped_swiglu(x, None, p8, off, n, a2, c2, ops.PHASE_DOWN))
+            ours["down_w8a16/random"] = 2.0 * n * h * inter / ms / 1e9
+        del x, w_gu, w_d, act, c2, a2
+        torch.cuda.empty_cache()
+    res["vendor_dense_bf16_gemm"] = vendor
+    res["grouped_kernel_one_group"] = ours
+    res["device"] = torch.cuda.get_device_name(0)
+    res["reps"] = reps
+    print(json.dumps(res))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="deepseek_v3_w8a16")
-    ap.add_argument("--all-workloads", action="store_true", help="one JSON line holding every synthetic workload")
+    ap.add_argument("--all-workloads", action="store_true", help="(default) every synthetic workload in the one JSON line")
+    ap.add_argument("--headline-only", action="store_true", help="only the workload named by --workload")
     ap.add_argument("--tokens", type=int, default=0, help="override the token count (parity/debug only)")
     ap.add_argument("--materialize", action="store_true", help="gather rows into a sorted copy instead of "
                     "reading them through the row map inside the GEMM")
@@ -297,19 +421,23 @@ def main():
     ap.add_argument("--staged", action="store_true", help="also time the block with weights staged from pinned host memory")
     ap.add_argument("--decoder-half", action="store_true", help="also time RMSNorm + block + residual add, fused and separate")
     ap.add_argument("--cpu-sample", type=int, default=1024, help="tokens of the workload the CPU baseline runs")
+    ap.add_argument("--ceiling", action="store_true", help="instead of the benchmark: registers-only MFMA rate, vendor dense "
+                    "bf16 GEMM and this library's one-group launch at the headline shapes, random and zero operands")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); use --gpus 1")
+    if args.ceiling:
+        return ceiling_run(args)
 
     import torch
     from moe_gen_amd import synthetic
     torch.cuda.set_device(0)
-    if args.all_workloads:
-        result = run_workload("deepseek_v3_w8a16", args, not args.no_cpu_baseline)
-        result["workloads"] = [run_workload(n, args, not args.no_cpu_baseline)
-                               for n in synthetic.WORKLOADS if n != "deepseek_v3_w8a16"]
-    else:
-        result = run_workload(args.workload, args, not args.no_cpu_baseline)
+    result = run_workload(args.workload, args, not args.no_cpu_baseline)
+    if not args.headline_only and args.workload == "deepseek_v3_w8a16" and not args.tokens:
+        # the other synthetic configurations: same steps / warm-up, each timed on its own
+        extra = argparse.Namespace(**{**vars(args), "staged": False, "decoder_half": False})
+        result["workloads"] = [run_workload(n, extra, not args.no_cpu_baseline)
+                               for n in synthetic.WORKLOADS if n != args.workload]
     print(json.dumps(result))
 
 

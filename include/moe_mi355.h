@@ -222,6 +222,24 @@ int moe_rmsnorm(const void* x, const void* weight, float eps, int32_t n_tokens, 
                 void* out, void* stream);
 
 /*
+ * moe_router reading its tokens THROUGH post_attention_layernorm (modeling_deepseek_v3.py:1361-1364:
+ * hidden_states = self.post_attention_layernorm(hidden_states); self.mlp(hidden_states) -> the gate's
+ * F.linear at :504-508): x holds the raw hidden states, each workgroup first computes the rstd of
+ * its tokens (moe_rmsnorm's summation order), normalises every chunk on its way to the matrix
+ * cores, xn = bf16(weight * bf16(f32(x) * rstd)), and writes the normalised rows once to x_norm
+ * for the expert GEMMs.  Results (x_norm, indices, weights, logits) are bit-identical to
+ * moe_rmsnorm followed by moe_router (with 32 experts or fewer, where the fused form does not pay,
+ * the call is those two launches).
+ *   x           device bf16 [n, h]  raw hidden states
+ *   norm_weight device bf16 [h]
+ *   x_norm      device bf16 [n, h]  out (must not alias x)
+ * Other arguments as moe_router.
+ */
+int moe_router_rmsnorm(const void* x, const void* norm_weight, float eps, const void* w_gate,
+                       const float* bias, const moe_router_params* params, void* x_norm,
+                       int32_t* topk_idx, float* topk_w, float* logits_out, void* stream);
+
+/*
  * moe_combine followed by the decoder layer's residual add
  * (hidden_states = residual + hidden_states, modeling_deepseek_v3.py:1365) in the same pass:
  *     out[t] = bf16( f32(residual[t]) + f32(<moe_combine result>[t]) )

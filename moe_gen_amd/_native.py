@@ -31,6 +31,8 @@ SIGNATURES = {
     "moe_version": (ctypes.c_char_p, []),
     "moe_router": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, ctypes.POINTER(RouterParams), c_void_p,
                                   c_void_p, c_void_p, c_void_p]),
+    "moe_router_rmsnorm": (ctypes.c_int, [c_void_p, c_void_p, ctypes.c_float, c_void_p, c_void_p,
+                                          ctypes.POINTER(RouterParams), c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "moe_dispatch_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32]),
     "moe_dispatch": (ctypes.c_int, [c_void_p, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p,
                                     c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_size_t, c_void_p]),

@@ -327,15 +327,16 @@ def moe_forward(block, hidden_states: torch.Tensor, spec: ops.RouterSpec, gate_w
     residual = None
     fuse = getattr(block, "_norm_residual", None)
     timer = getattr(block, "stage_timer", None)
-    if fuse is not None:                      # see norm_moe_residual
-        residual = x
-        with _span(timer, "rmsnorm"):
-            x = ops.rmsnorm(x, fuse[0], fuse[1])
     cache = block.__dict__.setdefault("_moe_cache", {})
     gw = _gate_weight_bf16(gate_weight, cache)
     b = None if bias is None else bias.data.to(torch.float32)
-    with _span(timer, "router"):
-        idx, w, logits = ops.router(x, gw, b, spec, want_logits)
+    if fuse is not None:                      # see norm_moe_residual: the router reads x through the norm
+        residual = x
+        with _span(timer, "router"):
+            idx, w, logits, x = ops.router(x, gw, b, spec, want_logits, norm_weight=fuse[0], eps=fuse[1])
+    else:
+        with _span(timer, "router"):
+            idx, w, logits = ops.router(x, gw, b, spec, want_logits)
     block.last_topk_idx, block.last_topk_weight = idx, w
     fused_gather = getattr(block, "fused_gather", True)
     with _span(timer, "dispatch"):
@@ -374,7 +375,8 @@ def norm_moe_residual(block, hidden_states: torch.Tensor, norm_weight: torch.Ten
         hidden_states = mlp(hidden_states)
         hidden_states = residual + hidden_states
 
-    with the norm as one kernel and the residual add folded into the combine's output pass.
+    with the norm folded into the router's read of the rows (its normalised copy is a side output
+    that the expert GEMMs read) and the residual add folded into the combine's output pass.
     Returns what `block(...)` returns with the new residual stream in place of the block output
     (Mixtral: a tuple with the router logits second)."""
     w = norm_weight.data if isinstance(norm_weight, torch.nn.Parameter) else norm_weight

@@ -30,6 +30,17 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
 }
 __device__ __forceinline__ float round_to_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
 
+// Two fp32 -> packed bf16 (a in the low half) with the hardware conversion v_cvt_pk_bf16_f32: round to
+// nearest even, NaN -> (bits >> 16) | 0x40, i.e. the same bits as f32_to_bf16_bits for every one of
+// the 2^32 inputs (checked exhaustively on the device).
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+    f32x2 f = {a, b};
+    bf16x2 h = __builtin_convertvector(f, bf16x2);
+    return __builtin_bit_cast(uint32_t, h);
+}
+
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
 }  // namespace moe

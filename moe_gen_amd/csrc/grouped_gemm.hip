@@ -48,14 +48,6 @@ constexpr int ROW_B = 128;       // bytes per LDS row
 constexpr int BN_ROWS = 256;     // weight rows per workgroup (128 gate + 128 up when SWIGLU)
 constexpr int MAX_E = 1024;
 
-typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2;
-typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
-
-__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
-    f32x2 f = {a, b};
-    bf16x2 h = __builtin_convertvector(f, bf16x2);  // v_cvt_pk_bf16_f32: round to nearest even
-    return __builtin_bit_cast(uint32_t, h);
-}
 __device__ __forceinline__ float bf16r(float a) { return __uint_as_float(pack_bf16(a, 0.0f) << 16); }
 
 // 16 fp8 bytes -> 16 bf16 (two 16-byte chunks): bf16(f32(q) * s)

@@ -49,17 +49,17 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const u32x4* __restrict__ 
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) acc = acc + __shfl_xor(acc, m);
     const float var = acc / (float)(chunks * 8);
-    const float rstd = 1.0f / __fsqrt_rn(var + eps);
+    // sqrt and divide correctly rounded: the plain operators are (the __fsqrt_rn intrinsic is the
+    // bare v_sqrt_f32, 1 ulp, and flips a bf16 rounding of x * rstd about once in a few hundred rows)
+    const float rstd = 1.0f / __builtin_sqrtf(var + eps);
     u32x4* orow = out + (size_t)row * chunks;
     auto scale = [&](const u32x4 v, const u32x4 g) {
         u32x4 o;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float lo = round_to_bf16(__uint_as_float(v[i] << 16) * rstd);
-            const float hi = round_to_bf16(__uint_as_float(v[i] & 0xffff0000u) * rstd);
-            const uint32_t a = f32_to_bf16_bits(__uint_as_float(g[i] << 16) * lo);
-            const uint32_t b = f32_to_bf16_bits(__uint_as_float(g[i] & 0xffff0000u) * hi);
-            o[i] = a | (b << 16);
+            const uint32_t y = pack_bf16(__uint_as_float(v[i] << 16) * rstd, __uint_as_float(v[i] & 0xffff0000u) * rstd);
+            o[i] = pack_bf16(__uint_as_float(g[i] << 16) * __uint_as_float(y << 16),
+                             __uint_as_float(g[i] & 0xffff0000u) * __uint_as_float(y & 0xffff0000u));
         }
         return o;
     };

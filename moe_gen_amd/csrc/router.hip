@@ -254,11 +254,24 @@ __device__ void route_token(const float* row, const float* __restrict__ bias, co
 //                  where 5 waves x 32 put two waves on one SIMD (128 cycles, as slow as 256 experts).
 // Global loads run two k-stages ahead in registers (two register sets, loop unrolled by two), which
 // is what hides the load latency when only a few workgroups exist (small token counts).
-template <bool SMALL, int TG, int NEB, int WE, int WT, int GW, int NX = 0>
+// NORM: the rows of x are raw hidden states and the router reads them through the decoder layer's
+//                  RMSNorm (post_attention_layernorm, modeling_deepseek_v3.py:125-150, call site :1363):
+//                  a pre-pass gives every token of the workgroup its rstd (one wave per row, the
+//                  summation order of rmsnorm_kernel), each staged chunk is normalised on its way to LDS,
+//                  xn = bf16(w * bf16(x * rstd)), and written once to nrm.out for the expert GEMMs.  The
+//                  memory pipe idles while the matrix cores run the logits, so the second read of the
+//                  rows and the side output cost little next to a separate norm kernel.
+struct NormArgs {
+    const uint16_t* w;   // [h] bf16, NULL: no norm
+    float eps;
+    uint16_t* out;       // [n, h] bf16 normalised rows
+};
+
+template <bool SMALL, int TG, int NEB, int WE, int WT, int GW, int NX, bool NORM>
 __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ wg, const float* __restrict__ bias,
     moe_router_params p, int32_t* __restrict__ topk_idx, float* __restrict__ topk_w,
-    float* __restrict__ logits_out) {
+    float* __restrict__ logits_out, NormArgs nrm) {
     constexpr int KC = SMALL ? 64 : 32;  // k elements per LDS stage
     constexpr int LDK = KC + 4;          // padded fp32 row stride: conflict-free 16-byte reads
     constexpr int NT = 64 * WE * WT;  // threads
@@ -282,7 +295,56 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     const int n = p.n_tokens, h = p.hidden, E = p.n_experts;
     const int t0 = blockIdx.x * BT;
 
-    u32x4 xr[2][XPT], wr[2][WPT];
+    __shared__ float s_rstd[NORM ? BT : 1];
+    if (NORM) {
+        // rstd of the block's tokens, one wave per row: lane l adds the squares of the 8-element chunks
+        // l, l+64, ... in ascending order, xor butterfly 32..1, var = sum / h, rstd = 1 / sqrt(var + eps)
+        const int chunks = h / 8;
+        for (int tb = wave; tb < BT; tb += NT / 64) {
+            const u32x4* row = reinterpret_cast<const u32x4*>(x + (size_t)min(t0 + tb, n - 1) * h);
+            float a = 0.0f;
+            for (int c0 = 0; c0 < chunks; c0 += 512) {   // 8 loads in flight per lane
+                u32x4 v[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[j] = row[min(c0 + lane + 64 * j, chunks - 1)];
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (c0 + lane + 64 * j < chunks) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const float lo = __uint_as_float(v[j][i] << 16), hi = __uint_as_float(v[j][i] & 0xffff0000u);
+                            a = a + lo * lo;
+                            a = a + hi * hi;
+                        }
+                    }
+            }
+#pragma unroll
+            for (int m = 32; m >= 1; m >>= 1) a = a + __shfl_xor(a, m);
+            const float var = a / (float)h;
+            if (lane == 0) s_rstd[tb] = 1.0f / __builtin_sqrtf(var + nrm.eps);
+        }
+        __syncthreads();
+    }
+
+    u32x4 xr[2][XPT], wr[2][WPT], gr[2][NORM ? XPT : 1];
+    float rstd_r[NORM ? XPT : 1];            // rstd of the token row behind this thread's i-th chunk
+    if (NORM) {
+#pragma unroll
+        for (int i = 0; i < XPT; ++i) rstd_r[i] = s_rstd[min((tid + i * NT) / (KC / 8), BT - 1)];
+    }
+    // Dword q (two elements) of chunk i of a register set, normalised in place:
+    // xn = bf16(w * bf16(x * rstd)), the rounding points of the reference's norm module, 12 vector
+    // instructions per pair with the packed hardware conversion.  The fp32 matrix instructions run on
+    // the same fp32 lanes as vector arithmetic, so this work is paid in logit time wherever it stands;
+    // the pieces are spread over the MFMAs of the stage before the one that stores the set so that at
+    // least no wave waits for another's.
+    auto norm_piece = [&](int set, int i, int q) {
+        const uint32_t xw = xr[set][i][q], gw = gr[set][i][q];
+        const float r = rstd_r[i];
+        const uint32_t y = pack_bf16(__uint_as_float(xw << 16) * r, __uint_as_float(xw & 0xffff0000u) * r);
+        xr[set][i][q] = pack_bf16(__uint_as_float(gw << 16) * __uint_as_float(y << 16),
+                                  __uint_as_float(gw & 0xffff0000u) * __uint_as_float(y & 0xffff0000u));
+    };
     // Loads are unconditional (addresses clamped; chunks beyond h are zeroed when they are stored
     // to LDS, two stages later): a load under a branch makes the compiler wait for ALL outstanding
     // loads before the first LDS store of a stage, and a select right after the load makes it
@@ -294,6 +356,7 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
             const int row = c / (KC / 8), kk = k0 + (c % (KC / 8)) * 8;
             const int t = min(t0 + row, n - 1);
             xr[set][i] = *reinterpret_cast<const u32x4*>(x + (size_t)t * h + (kk < h ? kk : 0));
+            if (NORM) gr[set][i] = *reinterpret_cast<const u32x4*>(nrm.w + (kk < h ? kk : 0));
         }
 #pragma unroll
         for (int i = 0; i < WPT; ++i) {
@@ -317,8 +380,14 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
 #pragma unroll
         for (int i = 0; i < XPT; ++i) {
             int c = tid + i * NT;
-            const bool ok = k0 + (c % (KC / 8)) * 8 < h;
-            if (c < XCH) store_chunk(Xs, c, ok ? xr[set][i] : u32x4{0, 0, 0, 0});
+            const int kk = k0 + (c % (KC / 8)) * 8;
+            const bool ok = kk < h;
+            const u32x4 v = xr[set][i];               // NORM: already normalised (norm_piece)
+            if (NORM && c < XCH) {
+                const int row = c / (KC / 8);
+                if (ok && t0 + row < n) *reinterpret_cast<u32x4*>(nrm.out + (size_t)(t0 + row) * h + kk) = v;
+            }
+            if (c < XCH) store_chunk(Xs, c, ok ? v : u32x4{0, 0, 0, 0});
         }
 #pragma unroll
         for (int i = 0; i < WPT; ++i) {
@@ -355,12 +424,17 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
             for (int j = 0; j < NX; ++j) b[2 + j] = *reinterpret_cast<const f32x4*>(bx_row + j * 4 * LDK + k4 * 4);
         }
     };
-    auto multiply_stage = [&]() {
+    constexpr int NPIECE = XPT * 4, PER_K4 = (NPIECE + KC / 4 - 1) / (KC / 4);
+    auto multiply_stage = [&](int nset) {    // nset: register set of the NEXT stage, normalised on the way (NORM)
         f32x4 a[2], b[2][NB4];
         read_ops(0, a[0], b[0]);
 #pragma unroll
         for (int k4 = 0; k4 < KC / 4; ++k4) {
             if (k4 + 1 < KC / 4) read_ops(k4 + 1, a[(k4 + 1) & 1], b[(k4 + 1) & 1]);
+            if (NORM) {
+#pragma unroll
+                for (int e = k4 * PER_K4; e < (k4 + 1) * PER_K4 && e < NPIECE; ++e) norm_piece(nset, e / 4, e % 4);
+            }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
@@ -386,11 +460,15 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     const int nstage = (h + KC - 1) / KC;
     load_stage(0, 0);
     load_stage(min(1, nstage - 1) * KC, 1);
+    if (NORM) {                              // the first stage has no stage before it to hide behind
+#pragma unroll
+        for (int e = 0; e < NPIECE; ++e) norm_piece(0, e / 4, e % 4);
+    }
     auto stage = [&](int st, int set) {      // set == st & 1, a literal at both call sites
         store_stage(set, st * KC);
         __syncthreads();
         load_stage(min(st + 2, nstage - 1) * KC, set);
-        multiply_stage();
+        multiply_stage(set ^ 1);             // (the other set holds stage st + 1, requested one stage ago)
         __syncthreads();
     };
     int st = 0;
@@ -453,11 +531,15 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
 
 template <bool SMALL, int TG, int NEB, int WE, int WT, int GW, int NX = 0>
 int launch(const void* x, const void* w, const float* bias, const moe_router_params& p, int32_t* idx,
-           float* tw, float* lo, hipStream_t st) {
+           float* tw, float* lo, const NormArgs& nrm, hipStream_t st) {
     constexpr int BT = SMALL ? 4 * TG * WT : 64 * WT;
     dim3 grid((p.n_tokens + BT - 1) / BT), block(64 * WE * WT);
-    hipLaunchKernelGGL((router_kernel<SMALL, TG, NEB, WE, WT, GW, NX>), grid, block, 0, st, (const uint16_t*)x,
-                       (const uint16_t*)w, bias, p, idx, tw, lo);
+    if (nrm.w)
+        hipLaunchKernelGGL((router_kernel<SMALL, TG, NEB, WE, WT, GW, NX, true>), grid, block, 0, st, (const uint16_t*)x,
+                           (const uint16_t*)w, bias, p, idx, tw, lo, nrm);
+    else
+        hipLaunchKernelGGL((router_kernel<SMALL, TG, NEB, WE, WT, GW, NX, false>), grid, block, 0, st, (const uint16_t*)x,
+                           (const uint16_t*)w, bias, p, idx, tw, lo, nrm);
     MOE_HIP_CHECK(hipGetLastError());
     return MOE_OK;
 }
@@ -465,9 +547,42 @@ int launch(const void* x, const void* w, const float* bias, const moe_router_par
 }  // namespace
 }  // namespace moe
 
+namespace moe {
+namespace {
+int route(const void* x, const void* w_gate, const float* bias, const moe_router_params* params, int32_t* topk_idx,
+          float* topk_w, float* logits_out, const NormArgs& nrm, void* stream);
+}
+}  // namespace moe
+
 extern "C" int moe_router(const void* x, const void* w_gate, const float* bias, const moe_router_params* params,
                           int32_t* topk_idx, float* topk_w, float* logits_out, void* stream) {
+    return moe::route(x, w_gate, bias, params, topk_idx, topk_w, logits_out, moe::NormArgs{nullptr, 0.0f, nullptr}, stream);
+}
+
+extern "C" int moe_router_rmsnorm(const void* x, const void* norm_weight, float eps, const void* w_gate,
+                                  const float* bias, const moe_router_params* params, void* x_norm,
+                                  int32_t* topk_idx, float* topk_w, float* logits_out, void* stream) {
     using namespace moe;
+    if (params != nullptr && params->n_tokens == 0) return MOE_OK;
+    MOE_REQUIRE(norm_weight && x_norm, "moe_router_rmsnorm: NULL norm weight or output");
+    MOE_REQUIRE(x_norm != x, "moe_router_rmsnorm: x_norm must not alias x (rows are read twice)");
+    MOE_REQUIRE(eps >= 0.0f, "moe_router_rmsnorm: eps %g < 0", (double)eps);
+    if (params != nullptr && params->n_experts <= 32) {
+        // Few experts: a launch is short chains of small MFMAs on few waves, with nothing to hide the
+        // per-workgroup pre-pass behind (Mixtral-8x7B, 16384 tokens: 0.149 ms fused against 0.088 +
+        // 0.045 ms).  The norm kernel followed by the plain router gives the same bits.
+        int rc = moe_rmsnorm(x, norm_weight, eps, params->n_tokens, params->hidden, x_norm, stream);
+        if (rc != MOE_OK) return rc;
+        return route(x_norm, w_gate, bias, params, topk_idx, topk_w, logits_out, NormArgs{nullptr, 0.0f, nullptr}, stream);
+    }
+    return route(x, w_gate, bias, params, topk_idx, topk_w, logits_out,
+                 NormArgs{static_cast<const uint16_t*>(norm_weight), eps, static_cast<uint16_t*>(x_norm)}, stream);
+}
+
+namespace moe {
+namespace {
+int route(const void* x, const void* w_gate, const float* bias, const moe_router_params* params, int32_t* topk_idx,
+          float* topk_w, float* logits_out, const NormArgs& nrm, void* stream) {
     MOE_REQUIRE(params != nullptr, "moe_router: params is NULL");
     const moe_router_params& p = *params;
     MOE_REQUIRE(p.n_tokens >= 0, "moe_router: n_tokens %d < 0", p.n_tokens);
@@ -494,7 +609,7 @@ extern "C" int moe_router(const void* x, const void* w_gate, const float* bias, 
     hipStream_t st = as_stream(stream);
     const int E = p.n_experts, n = p.n_tokens;
 #define MOE_ROUTE(SMALL, TG, NEB, WE, WT, GW) \
-    return launch<SMALL, TG, NEB, WE, WT, GW>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st)
+    return launch<SMALL, TG, NEB, WE, WT, GW>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, nrm, st)
     // The 4x4 engine's 16 blocks per instruction are laid out as 64 tokens x 4 experts, 16 x 16 or
     // 4 x 64: the fewer tokens a launch has, the fewer go to a workgroup, so that the sequential-in-k
     // chains run on as many CUs as possible; many tokens take the 32x32 engine (an eighth of the LDS
@@ -538,7 +653,7 @@ extern "C" int moe_router(const void* x, const void* w_gate, const float* bias, 
     // many tokens, more than 64 experts: one wave per 32 experts (one MFMA per k and wave, no padding
     // beyond the next multiple of 32) measured 10-25 % faster than half as many waves with two MFMAs each
 #define MOE_ROUTE_X(WE, NX) \
-    return launch<false, 16, 1, WE, 1, 64, NX>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st)
+    return launch<false, 16, 1, WE, 1, 64, NX>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, nrm, st)
     if (E <= 96) MOE_ROUTE(false, 16, 1, 3, 1, 64);
     if (E <= 128) MOE_ROUTE(false, 16, 1, 4, 1, 64);
     // Between 4 and 8 waves' worth of experts: 4 waves x (32 + 4 NX) keep the four SIMDs evenly loaded,
@@ -555,3 +670,5 @@ extern "C" int moe_router(const void* x, const void* w_gate, const float* bias, 
 #undef MOE_ROUTE_X
 #undef MOE_ROUTE
 }
+}  // namespace
+}  // namespace moe

@@ -51,9 +51,14 @@ def _need(t: torch.Tensor, dtype, name: str, shape=None):
         raise ValueError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
 
 
-def router(x: torch.Tensor, gate_w: torch.Tensor, bias, spec: RouterSpec, want_logits: bool = False):
+def router(x: torch.Tensor, gate_w: torch.Tensor, bias, spec: RouterSpec, want_logits: bool = False,
+           norm_weight: torch.Tensor | None = None, eps: float = 1e-6):
     """x bf16 [n,h], gate_w bf16 [E,h], bias fp32 [E] | None ->
-    (topk_idx int32 [n,k], topk_weight fp32 [n,k], logits fp32 [n,E] | None)."""
+    (topk_idx int32 [n,k], topk_weight fp32 [n,k], logits fp32 [n,E] | None).
+
+    With norm_weight (bf16 [h]) the rows of x are raw hidden states read through the decoder
+    layer's RMSNorm inside the same kernel, and a fourth result holds the normalised rows
+    (bf16 [n,h]) -- bit-identical to rmsnorm() followed by router()."""
     n, h = x.shape
     E, k = spec.n_experts, spec.top_k
     _need(x, torch.bfloat16, "x")
@@ -73,6 +78,13 @@ def router(x: torch.Tensor, gate_w: torch.Tensor, bias, spec: RouterSpec, want_l
                        METHOD[spec.method], int(spec.norm_topk_prob), spec.scale_mode,
                        int(spec.logits_bf16), int(spec.weights_bf16), spec.norm_eps,
                        spec.routed_scaling_factor)
+    if norm_weight is not None:
+        _need(norm_weight, torch.bfloat16, "norm weight", (h,))
+        xn = torch.empty_like(x)
+        N.check(N.lib().moe_router_rmsnorm(_ptr(x), _ptr(norm_weight), float(eps), _ptr(gate_w), _ptr(bias),
+                                           ctypes.byref(p), _ptr(xn), _ptr(idx), _ptr(w), _ptr(lg), _stream()),
+                "moe_router_rmsnorm")
+        return idx, w, lg, xn
     N.check(N.lib().moe_router(_ptr(x), _ptr(gate_w), _ptr(bias), ctypes.byref(p), _ptr(idx), _ptr(w),
                                _ptr(lg), _stream()), "moe_router")
     return idx, w, lg
