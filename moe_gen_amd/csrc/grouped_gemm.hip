@@ -103,6 +103,59 @@ __device__ __forceinline__ const uint8_t* uni_ptr(const void* p) {
     return reinterpret_cast<const uint8_t*>((uintptr_t)(((uint64_t)hi << 32) | lo));
 }
 
+
+// ---- pieces shared by the one-workgroup-per-tile kernel and the persistent kernel ----
+
+// Position of the expert's `local`-th tile.  Inside an expert, tiles are visited in groups of about
+// GM consecutive M tiles (the expert's M tiles split as evenly as possible); within a group the M
+// tile varies fastest.  The ~32 workgroups an XCD runs at once then cover ~GM M tiles x 32/GM N
+// tiles and share those panels through the XCD's L2: an A panel is fetched once per 32/GM N tiles
+// and a B panel once per group.  GM = 4 (4 x 8 tiles) balances the two re-fetch factors; measured on
+// 64 experts x 2048 rows (7168 -> 2048, fp8) it fetches 7.0 GiB against 8.75 GiB for GM = 8 or 16.
+__device__ __forceinline__ void tile_in_expert(int local, int mt_e, int n_tiles_n, int& m_tile, int& n_tile) {
+    constexpr int GM = 4;
+    const int ng = max(1, (mt_e + GM / 2) / GM);
+    const int base = mt_e / ng, extra = mt_e - base * ng;      // `extra` groups hold base+1 tiles
+    const int big = (base + 1) * n_tiles_n, cut = extra * big;
+    int gm, m0, rem;
+    if (local < cut) {
+        const int gi = local / big;
+        rem = local - gi * big; gm = base + 1; m0 = gi * (base + 1);
+    } else {
+        const int l2 = local - cut, sz = base * n_tiles_n, gi = l2 / sz;
+        rem = l2 - gi * sz; gm = base; m0 = extra * (base + 1) + gi * base;
+    }
+    n_tile = rem / gm;
+    m_tile = m0 + (rem - n_tile * gm);
+}
+
+// 8 fp8 weights (two dwords) -> 8 bf16: bf16(f32(q) * s), the reference's dequantisation
+__device__ __forceinline__ u32x4 dequant8(uint32_t q0, uint32_t q1, float sc) {
+    const f32x2 c0 = __builtin_amdgcn_cvt_pk_f32_fp8(q0, false), c1 = __builtin_amdgcn_cvt_pk_f32_fp8(q0, true);
+    const f32x2 c2 = __builtin_amdgcn_cvt_pk_f32_fp8(q1, false), c3 = __builtin_amdgcn_cvt_pk_f32_fp8(q1, true);
+    return u32x4{pack_bf16(c0[0] * sc, c0[1] * sc), pack_bf16(c1[0] * sc, c1[1] * sc),
+                 pack_bf16(c2[0] * sc, c2[1] * sc), pack_bf16(c3[0] * sc, c3[1] * sc)};
+}
+
+// Epilogue values of one lane for one pair of accumulators: 4 consecutive output columns of one row.
+// SWIGLU: act = bf16(bf16(silu(bf16(g))) * bf16(u)), the rounding points of the reference's bf16
+// Linear / SiLU / mul modules (silu through the hardware exp and reciprocal); else bf16(acc).
+template <bool SWIGLU>
+__device__ __forceinline__ u32x2 epilogue_pack(const f32x4& a, const f32x4& up) {
+    if (SWIGLU) {
+        float o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float gv = bf16r(a[i]);
+            const float uv = bf16r(up[i]);
+            const float sg = bf16r(gv * __builtin_amdgcn_rcpf(1.0f + __expf(-gv)));
+            o[i] = sg * uv;
+        }
+        return u32x2{pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3])};
+    }
+    return u32x2{pack_bf16(a[0], a[1]), pack_bf16(a[2], a[3])};
+}
+
 // MT: 32-row units per wave along M (workgroup rows BM = 64*MT, 2 waves along M)
 // WN: waves along N; 4 -> 8 waves of up to 128x64 outputs, two per SIMD; every wave interleaves
 //     its share of the load / dequantise / LDS-store work with its MFMAs, a piece per MFMA group
@@ -194,26 +247,8 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     const int e = uni(s_sel[0]);
     const int pe = uni(s_sel[1]);
     const int mt_e = uni(s_sel[2]);
-    // Inside an expert, tiles are visited in groups of about GM consecutive M tiles (the expert's
-    // M tiles split as evenly as possible); within a group the M tile varies fastest.  The ~32
-    // workgroups an XCD runs at once then cover ~GM M tiles x 32/GM N tiles and share those
-    // panels through the XCD's L2: an A panel is fetched once per 32/GM N tiles and a B panel
-    // once per group.  GM = 4 (4 x 8 tiles) balances the two re-fetch factors; measured on 64
-    // experts x 2048 rows (7168 -> 2048, fp8) it fetches 7.0 GiB against 8.75 GiB for GM = 8 or 16.
-    constexpr int GM = 4;
-    const int local = v - pe * g.n_tiles_n;
-    const int ng = max(1, (mt_e + GM / 2) / GM);
-    const int base = mt_e / ng, extra = mt_e - base * ng;      // `extra` groups hold base+1 tiles
-    const int big = (base + 1) * g.n_tiles_n, cut = extra * big;
-    int gm, m0, rem;
-    if (local < cut) {
-        const int gi = local / big;
-        rem = local - gi * big; gm = base + 1; m0 = gi * (base + 1);
-    } else {
-        const int l2 = local - cut, sz = base * g.n_tiles_n, gi = l2 / sz;
-        rem = l2 - gi * sz; gm = base; m0 = extra * (base + 1) + gi * base;
-    }
-    const int n_tile = rem / gm, m_tile = m0 + (rem - n_tile * gm);
+    int m_tile, n_tile;
+    tile_in_expert(v - pe * g.n_tiles_n, mt_e, g.n_tiles_n, m_tile, n_tile);
     const int row0 = uni(s_sel[3]) + m_tile * BM;
     const int row_end = uni(s_sel[4]);
     const int n0 = n_tile * NBLK;
@@ -392,11 +427,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
             const int b = (i - NA) >> 1, half = (i - NA) & 1;
             const uint8_t* m = (SWIGLU && b >= NB / 2) ? bmat1 : bmat0;
             const float sc = rs[set][b / (NB / 2)];
-            const uint32_t q0 = rb[set][b][2 * half], q1 = rb[set][b][2 * half + 1];
-            const f32x2 c0 = __builtin_amdgcn_cvt_pk_f32_fp8(q0, false), c1 = __builtin_amdgcn_cvt_pk_f32_fp8(q0, true);
-            const f32x2 c2 = __builtin_amdgcn_cvt_pk_f32_fp8(q1, false), c3 = __builtin_amdgcn_cvt_pk_f32_fp8(q1, true);
-            const u32x4 o = {pack_bf16(c0[0] * sc, c0[1] * sc), pack_bf16(c1[0] * sc, c1[1] * sc),
-                             pack_bf16(c2[0] * sc, c2[1] * sc), pack_bf16(c3[0] * sc, c3[1] * sc)};
+            const u32x4 o = dequant8(rb[set][b][2 * half], rb[set][b][2 * half + 1], sc);
             // the first 8 weights go to b_lds[0], the second 8 to b_lds[1]; swapped rows the other way round
             *reinterpret_cast<u32x4*>(Bs + ((half ^ (b_swap ? 1 : 0)) ? b_lds[1] : b_lds[0]) + b * RB * ROW_B) = o;
             if (half == 1) {
@@ -476,20 +507,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
         const int key = (r >> KSH) & (CPR - 1);
 #pragma unroll
         for (int jj = 0; jj < (SWIGLU ? TN / 2 : TN); ++jj) {
-            u32x2 pk;
-            if (SWIGLU) {
-                float o[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    float gv = bf16r(acc[mi][jj][i]);
-                    float uv = bf16r(acc[mi][jj + TN / 2][i]);
-                    float sg = bf16r(gv * __builtin_amdgcn_rcpf(1.0f + __expf(-gv)));
-                    o[i] = sg * uv;
-                }
-                pk = u32x2{pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3])};
-            } else {
-                pk = u32x2{pack_bf16(acc[mi][jj][0], acc[mi][jj][1]), pack_bf16(acc[mi][jj][2], acc[mi][jj][3])};
-            }
+            const u32x2 pk = epilogue_pack<SWIGLU>(acc[mi][jj], acc[mi][SWIGLU ? jj + TN / 2 : jj]);
             *reinterpret_cast<u32x2*>(erow + (((2 * jj + (fquad >> 1)) ^ key) << 4)) = pk;
         }
     }
@@ -553,7 +571,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
 
     // ---- M-tile prefix over experts (exclusive scan of ceil(count/BM)) ----
     int run = 0;
-    int my_start = 0, my_mt = 0, my_o0 = 0, my_o1 = 0;   // this thread's expert (of the last pass)
+    int my_start = 0, my_o0 = 0, my_o1 = 0;   // this thread's expert (of the last pass)
     for (int e0 = 0; e0 < g.E; e0 += NT) {
         int e = e0 + tid;
         int mt = 0;
@@ -583,7 +601,6 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
             tot += s_wtot[w];
         }
         my_start = pre + inc - mt;
-        my_mt = mt;
         if (e < g.E) s_pref[e] = my_start;
         run += tot;
         if (g.E > NT) __syncthreads();   // s_wtot is rewritten by the next pass
@@ -624,26 +641,8 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
     const int e = cur_e;
     const int pe = uni(s_pref[e]);
     const int mt_e = uni(s_pref[e + 1]) - pe;
-    // Inside an expert, tiles are visited in groups of about GM consecutive M tiles (the expert's
-    // M tiles split as evenly as possible); within a group the M tile varies fastest.  The ~32
-    // workgroups an XCD runs at once then cover ~GM M tiles x 32/GM N tiles and share those
-    // panels through the XCD's L2: an A panel is fetched once per 32/GM N tiles and a B panel
-    // once per group.  GM = 4 (4 x 8 tiles) balances the two re-fetch factors; measured on 64
-    // experts x 2048 rows (7168 -> 2048, fp8) it fetches 7.0 GiB against 8.75 GiB for GM = 8 or 16.
-    constexpr int GM = 4;
-    const int local = v - pe * g.n_tiles_n;
-    const int ng = max(1, (mt_e + GM / 2) / GM);
-    const int base = mt_e / ng, extra = mt_e - base * ng;      // `extra` groups hold base+1 tiles
-    const int big = (base + 1) * g.n_tiles_n, cut = extra * big;
-    int gm, m0, rem;
-    if (local < cut) {
-        const int gi = local / big;
-        rem = local - gi * big; gm = base + 1; m0 = gi * (base + 1);
-    } else {
-        const int l2 = local - cut, sz = base * g.n_tiles_n, gi = l2 / sz;
-        rem = l2 - gi * sz; gm = base; m0 = extra * (base + 1) + gi * base;
-    }
-    const int n_tile = rem / gm, m_tile = m0 + (rem - n_tile * gm);
+    int m_tile, n_tile;
+    tile_in_expert(v - pe * g.n_tiles_n, mt_e, g.n_tiles_n, m_tile, n_tile);
     row0 = uni(s_off[e]) + m_tile * BM;
     row_end = uni(s_off[e + 1]);
     n0 = n_tile * NBLK;
@@ -802,11 +801,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
         } else if (W8) {
             const int b = (i - NA) >> 1, half = (i - NA) & 1;
             const float sc = rs[set][b / (NB / 2)];
-            const uint32_t q0 = rb[set][b][2 * half], q1 = rb[set][b][2 * half + 1];
-            const f32x2 c0 = __builtin_amdgcn_cvt_pk_f32_fp8(q0, false), c1 = __builtin_amdgcn_cvt_pk_f32_fp8(q0, true);
-            const f32x2 c2 = __builtin_amdgcn_cvt_pk_f32_fp8(q1, false), c3 = __builtin_amdgcn_cvt_pk_f32_fp8(q1, true);
-            const u32x4 o = {pack_bf16(c0[0] * sc, c0[1] * sc), pack_bf16(c1[0] * sc, c1[1] * sc),
-                             pack_bf16(c2[0] * sc, c2[1] * sc), pack_bf16(c3[0] * sc, c3[1] * sc)};
+            const u32x4 o = dequant8(rb[set][b][2 * half], rb[set][b][2 * half + 1], sc);
             // the first 8 weights go to b_lds[0], the second 8 to b_lds[1]; swapped rows the other way round
             *reinterpret_cast<u32x4*>(Bs + ((half ^ (b_swap ? 1 : 0)) ? b_lds[1] : b_lds[0]) + b * RB * ROW_B) = o;
             if (half == 1) {
@@ -925,20 +920,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
                 const int key = (r >> KSH) & (CPR - 1);
 #pragma unroll
                 for (int jj = 0; jj < (SWIGLU ? TN / 2 : TN); ++jj) {
-                    u32x2 pk;
-                    if (SWIGLU) {
-                        float o[4];
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            float gv = bf16r(acc[mi][jj][i]);
-                            float uv = bf16r(acc[mi][jj + TN / 2][i]);
-                            float sg = bf16r(gv * __builtin_amdgcn_rcpf(1.0f + __expf(-gv)));
-                            o[i] = sg * uv;
-                        }
-                        pk = u32x2{pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3])};
-                    } else {
-                        pk = u32x2{pack_bf16(acc[mi][jj][0], acc[mi][jj][1]), pack_bf16(acc[mi][jj][2], acc[mi][jj][3])};
-                    }
+                    const u32x2 pk = epilogue_pack<SWIGLU>(acc[mi][jj], acc[mi][SWIGLU ? jj + TN / 2 : jj]);
                     *reinterpret_cast<u32x2*>(erow + (((2 * jj + (efquad >> 1)) ^ key) << 4)) = pk;
                 }
             }

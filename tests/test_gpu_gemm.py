@@ -192,3 +192,52 @@ def test_dequant_golden_fixture():
     z = np.load(os.path.join(os.path.dirname(__file__), "golden", "fp8_dequant.npz"))
     out = ops.dequant_fp8_block128(torch.from_numpy(z["q"]).cuda().view(torch.float8_e4m3fn), torch.from_numpy(z["scale"]).cuda())
     assert np.array_equal(bits(out), z["out"])
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_swiglu_epilogue_alone(fp8):
+    """The SiLU*mul epilogue pinned on its own: one-hot token rows make every gate and up output a
+    single exact product, g[r,c] = Wg[c, r], u[r,c] = Wu[c, r], so `act` (the gate/up launch's
+    output) must be bf16(bf16(silu(g)) * u) -- torch's own bf16 silu and bf16 mul on the CPU are the
+    witness.  The kernel evaluates silu with the hardware exp and reciprocal (about 1e-6 relative),
+    so bf16(silu(g)) may land on the other side of a rounding boundary on a few elements: one bf16
+    step there, which the product with u turns into at most two steps of the result (a factor at the
+    bottom of its binade, a product at the top of one).  A swapped gate/up role, a missing rounding
+    point or a wrong sign fails everywhere."""
+    from moe_gen_amd import ops
+    from moe_gen_amd.synthetic import quantize_fp8_block128
+    h = I = 128
+    n = 3 * h                                            # every one-hot row three times, with different scales
+    g = torch.Generator().manual_seed(17)
+    if fp8:                                              # exactly representable after block quantisation: powers of two times small integers
+        wg = (torch.randint(-12, 13, (I, h), generator=g).float() * 0.25)
+        wu = (torch.randint(-8, 9, (I, h), generator=g).float() * 0.5)
+        wg[0, 0], wu[0, 0] = 28.0, 14.0                 # fixes each block's scale: amax = 28 -> 28/448 = 2^-4, 14/448 = 2^-5
+        qg, qu = quantize_fp8_block128(wg), quantize_fp8_block128(wu)
+        wg_f = torch.from_numpy(O.bf16_to_f32(O.dequant_block(bits(qg[0]), qg[1].numpy())))
+        wu_f = torch.from_numpy(O.bf16_to_f32(O.dequant_block(bits(qu[0]), qu[1].numpy())))
+        assert torch.equal(wg_f, wg) and torch.equal(wu_f, wu)
+        qd = quantize_fp8_block128(torch.zeros(h, I))
+        ptrs = ops.expert_pointers([qg[0].cuda()], [qu[0].cuda()], [qd[0].cuda()], [qg[1].cuda()], [qu[1].cuda()], [qd[1].cuda()])
+    else:
+        wg = (torch.randn(I, h, generator=g) * 4).to(torch.bfloat16)
+        wu = (torch.randn(I, h, generator=g) * 2).to(torch.bfloat16)
+        wg_f, wu_f = wg.float(), wu.float()
+        ptrs = ops.expert_pointers([wg.cuda()], [wu.cuda()], [torch.zeros(h, I, dtype=torch.bfloat16).cuda()])
+    scales = torch.tensor([1.0, 0.5, 4.0])
+    x = torch.zeros(n, h, dtype=torch.bfloat16)
+    for r in range(n):
+        x[r, r % h] = scales[r // h]
+    act = torch.empty(n, I, dtype=torch.bfloat16, device="cuda")
+    y = torch.empty(n, h, dtype=torch.bfloat16, device="cuda")
+    off = torch.tensor([0, n], dtype=torch.int32, device="cuda")
+    ops.grouped_swiglu(x.cuda(), None, ptrs, off, n, act, y, ops.PHASE_GATE_UP)
+    torch.cuda.synchronize()
+    gate = torch.stack([wg_f[:, r % h] * scales[r // h] for r in range(n)]).to(torch.bfloat16)   # exact: one product
+    up = torch.stack([wu_f[:, r % h] * scales[r // h] for r in range(n)]).to(torch.bfloat16)
+    want = torch.nn.functional.silu(gate) * up                                                    # bf16 modules, as the reference
+    got_bits, want_bits = bits(act).astype(np.int32), bits(want).astype(np.int32)
+    diff = np.abs(got_bits - want_bits)
+    assert diff.max() <= 2, f"epilogue off by {diff.max()} bf16 steps"
+    assert (diff > 0).mean() < 0.01, f"{(diff > 0).mean():.2%} of the elements differ"
+    assert (diff > 1).mean() < 0.001, f"{(diff > 1).mean():.3%} of the elements differ by two steps"
