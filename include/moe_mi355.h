@@ -136,6 +136,9 @@ int moe_dispatch_static(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k
  * on bf16 MFMA with fp32 accumulation.
  *   x         device bf16: rows of the sorted token matrix [n_rows, h]; or, when
  *             row_map != NULL, the unsorted matrix, row r being x[row_map[r]]
+ *   x_rows    rows of x (>= 1).  It bounds the gather: a row_map entry outside [0, x_rows) reads a row
+ *             of zeros where the descriptor-based loads are used (x smaller than 4 GiB) and is
+ *             undefined otherwise; without row_map it only has to cover the rows the call reads
  *   row_map   device int32 [n_rows] or NULL
  *   w_gate/w_up/w_down   device arrays of E device pointers: Wg_e, Wu_e bf16
  *             [I, h]; Wd_e bf16 [h, I]  (nn.Linear [out, in] layout)
@@ -154,7 +157,7 @@ int moe_dispatch_static(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k
  */
 enum { MOE_PHASE_GATE_UP = 1, MOE_PHASE_DOWN = 2, MOE_PHASE_BOTH = 3 };
 size_t moe_grouped_workspace_bytes(int32_t n_rows, int32_t n_experts);
-int moe_grouped_swiglu_bf16(const void* x, const int32_t* row_map,
+int moe_grouped_swiglu_bf16(const void* x, int32_t x_rows, const int32_t* row_map,
                             const void* const* w_gate, const void* const* w_up,
                             const void* const* w_down, const int32_t* offsets,
                             int32_t n_rows, int32_t n_experts, int32_t hidden, int32_t inter,
@@ -169,7 +172,7 @@ int moe_grouped_swiglu_bf16(const void* x, const int32_t* row_map,
  *   s_down       device array  of E pointers to fp32 [ceil(h/128), ceil(I/128)]
  * Requires h % 128 == 0 and I % 128 == 0.
  */
-int moe_grouped_swiglu_w8a16(const void* x, const int32_t* row_map,
+int moe_grouped_swiglu_w8a16(const void* x, int32_t x_rows, const int32_t* row_map,
                              const void* const* w_gate, const void* const* w_up,
                              const void* const* w_down,
                              const float* const* s_gate, const float* const* s_up,

@@ -39,10 +39,10 @@ SIGNATURES = {
     "moe_dispatch_static": (ctypes.c_int, [c_void_p, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p,
                                            c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p]),
     "moe_grouped_workspace_bytes": (c_size_t, [c_int32, c_int32]),
-    "moe_grouped_swiglu_bf16": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+    "moe_grouped_swiglu_bf16": (ctypes.c_int, [c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                                c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p,
                                                c_int32, c_void_p, c_size_t, c_void_p]),
-    "moe_grouped_swiglu_w8a16": (ctypes.c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+    "moe_grouped_swiglu_w8a16": (ctypes.c_int, [c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                                 c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32,
                                                 c_int32, c_void_p, c_void_p, c_int32, c_void_p, c_size_t, c_void_p]),
     "moe_dequant_fp8_block128": (ctypes.c_int, [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p]),

@@ -32,7 +32,8 @@
 // XOR swizzle so that both the 16-byte stores and the 16-byte MFMA operand reads are
 // bank-conflict free.  Global loads for tile k+2 are in flight while tile k is multiplied
 // and tile k+1 is written to LDS; every wave interleaves its share of that data movement with
-// its MFMAs, one piece per group of MFMAs, between the one barrier per k-stage.
+// its MFMAs, one piece per group of MFMAs, between the one barrier per k-stage.  The persistent
+// kernel brings token rows and bf16 weights into LDS by DMA instead (buffer_load ... lds).
 //
 // The MFMA is issued with the WEIGHT fragment as srcA and the TOKEN fragment as srcB, so
 // a lane ends up holding 4 consecutive output columns of one token row per accumulator;
@@ -65,6 +66,7 @@ __device__ __forceinline__ void dequant16(u32x4 q, float s, u32x4& lo, u32x4& hi
 struct GemmArgs {
     const uint16_t* a;          // activations, row stride K
     const int32_t* row_map;     // optional: sorted row -> row of a
+    size_t a_bytes;             // size of a when rows are gathered through row_map
     const void* const* b0;      // per-expert weight matrix [N, K] (gate when SWIGLU, else down)
     const void* const* b1;      // per-expert up matrix [N, K] (SWIGLU only)
     const float* const* s0;     // per-expert block scales of b0 (W8 only)
@@ -538,44 +540,59 @@ __device__ __forceinline__ int fresh_lane() {
     return l;
 }
 
-// Persistent variant of the BM = 256 kernel: one workgroup per CU walks its share of the tiles, and
-// the software pipeline runs on across the tile boundary: the last two
-// k-iterations of a tile already fetch the next tile's first two k-stages, the epilogue goes
-// through a small scratch of its own instead of the stages, and the next tile starts with its
-// first stage in LDS and its second in flight.  What a fresh workgroup pays per tile -- launch,
-// tile-prefix scan, pointer chase, first fetch, store drain: 6-8 us against 57 us of k loop for
-// K = 2048 -- is paid once per workgroup, or overlaps the previous tile's work.
+// Persistent kernel for BM = 256: one workgroup per CU walks its share of the tiles, and the software
+// pipeline runs on across the tile boundary (a tile's last k-iterations already fetch the next tile's
+// first stages, the epilogue goes through the idle stage, and the next tile starts with its first stage
+// in LDS).  What a fresh workgroup pays per tile -- launch, tile-prefix scan, pointer chase, first fetch,
+// store drain: 6-8 us against 57 us of k loop for K = 2048 -- is paid once per workgroup or overlaps
+// the previous tile's work.
+//
+// Token rows (and bf16 weights) reach LDS by DMA: buffer_load_dwordx4 ... lds writes 64 lanes x 16 bytes
+// to 1 KiB of consecutive LDS, each lane fetching the 16 bytes that belong at its position of the
+// swizzled layout, so there are no staging registers, no LDS store instructions and no per-chunk load
+// waits in the MFMA stream: a wave waits once per k-iteration, before the barrier, for its own DMA of the
+// next stage.  fp8 weights still go through registers (they are converted on the way), two k-stages
+// ahead.  Three things make this worth it (the same loads issued as global_load ... lds in one array per
+// stage measured 2 % slower than register staging; this form 3-5 % faster):
+//  * buffer (MUBUF) loads.  The compiler models the FLAT-encoded global_load ... lds as a possible LDS
+//    access through the flat aperture and from then on waits for ALL outstanding LDS operations
+//    (lgkmcnt(0)) wherever an operand fragment is needed, which serialises the fragment reads.
+//  * token stages and weight stages are separate LDS arrays.  An LDS store that may alias the target of
+//    an outstanding DMA gets a vmcnt(0) in front of it; the fp8 weight stores must not.
+//  * stage parities are literals (the k loop is unrolled by two), so reads of one stage provably do not
+//    alias the DMA into the other.
+typedef __attribute__((address_space(3))) uint8_t* lds_u8;
 template <bool SWIGLU, bool W8>
 __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g) {
     constexpr int MT = 4, WN = 4;
-    constexpr int NT = 128 * WN;                // threads
-    constexpr int BM = 64 * MT;                 // rows per workgroup
-    constexpr int A_STAGE = BM * ROW_B;         // bytes
+    constexpr int NT = 128 * WN;
+    constexpr int BM = 64 * MT;
+    constexpr int A_STAGE = BM * ROW_B;
     constexpr int B_STAGE = BN_ROWS * ROW_B;
-    constexpr int RA = NT / 8;                  // A rows covered by one pass of the workgroup
-    constexpr int NA = BM / RA;                 // 16-byte A chunks per thread per stage
-    constexpr int RB = W8 ? NT / 4 : NT / 8;    // B rows per pass (fp8 rows are 4 chunks of 16 weights)
-    constexpr int NB = BN_ROWS / RB;            // 16-byte global B chunks per thread per stage
-    constexpr int NBLK = SWIGLU ? 128 : 256;    // output columns per workgroup
-    constexpr int NJ = 8 / WN;                  // 32-row units of the weight tile per wave
-    static_assert(NA >= 1 && NB >= 2, "tile/thread mismatch");
-    // two separate arrays: stores into one stage and reads from the other provably do not alias,
-    // which lets the scheduler move them past each other
-    __shared__ __attribute__((aligned(16))) uint8_t smem0[A_STAGE + B_STAGE];
-    __shared__ __attribute__((aligned(16))) uint8_t smem1[A_STAGE + B_STAGE];
+    constexpr int RB = NT / 4;                  // fp8: B rows per pass (rows are 4 chunks of 16 weights)
+    constexpr int NB = BN_ROWS / RB;            // fp8: 16-byte global B chunks per thread per stage (2)
+    constexpr int NBLK = SWIGLU ? 128 : 256;
+    constexpr int NJ = 8 / WN;
+    constexpr int ND = 4;                       // DMA instructions per wave and tile half (32 rows of 128 bytes = 4 x 1 KiB)
+    // four separate arrays: the DMA writes the token stages, the fp8 path writes the weight stages with
+    // ordinary LDS stores; as separate objects the two provably do not alias (otherwise every LDS store
+    // waits for all outstanding DMA)
+    __shared__ __attribute__((aligned(1024))) uint8_t sA0[A_STAGE];
+    __shared__ __attribute__((aligned(1024))) uint8_t sA1[A_STAGE];
+    __shared__ __attribute__((aligned(1024))) uint8_t sB0[B_STAGE];
+    __shared__ __attribute__((aligned(1024))) uint8_t sB1[B_STAGE];
     __shared__ int s_pref[MAX_E + 1];
     __shared__ int s_wtot[NT / 64];
-    constexpr int PE = 512;                               // experts this kernel keeps tables for (18 KiB of LDS)
+    constexpr int PE = 512;
     __shared__ int s_off[PE + 1];
-    __shared__ unsigned long long s_ptr[4][PE];           // b0, b1, s0, s1 per expert
+    __shared__ unsigned long long s_ptr[4][PE];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wave_s = uni(wave);                         // scalar copy
+    const int wave_s = uni(wave);
     const int wm = wave_s & 1, wn = (wave_s >> 1) % WN;
 
-    // ---- M-tile prefix over experts (exclusive scan of ceil(count/BM)) ----
     int run = 0;
-    int my_start = 0, my_o0 = 0, my_o1 = 0;   // this thread's expert (of the last pass)
+    int my_start = 0, my_o0 = 0, my_o1 = 0;
     for (int e0 = 0; e0 < g.E; e0 += NT) {
         int e = e0 + tid;
         int mt = 0;
@@ -607,139 +624,147 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
         my_start = pre + inc - mt;
         if (e < g.E) s_pref[e] = my_start;
         run += tot;
-        if (g.E > NT) __syncthreads();   // s_wtot is rewritten by the next pass
+        if (g.E > NT) __syncthreads();
     }
     if (tid == 0) s_pref[g.E] = run;
     __syncthreads();
     const int total = run * g.n_tiles_n;
-
-    // ---- XCD-aware ids.  The `slots` workgroups of an XCD (= blockIdx % 8) work on `slots`
-    // consecutive tiles at a time (4 M tiles x 8 N tiles of one expert, sharing panels through the
-    // XCD's L2), and such groups go round-robin to the XCDs: group G belongs to XCD G % 8, so at any
-    // time the chip works on 8 neighbouring groups -- one or two experts -- whose panels the 256 MiB
-    // memory-side cache then holds for the other XCDs (each XCD on a far-apart range of its own:
-    // headline +2.5 %, Mixtral-8x7B +2.7 % slower).  The workgroup in slot c of its XCD takes tile c
-    // of the XCD's 1st, 2nd, ... group.
     const int xcd = blockIdx.x & 7, slots = gridDim.x >> 3;
     int slot = blockIdx.x >> 3;
     auto tile_of = [&](int sl) { return ((sl / slots) * 8 + xcd) * slots + (sl % slots); };
     if (tile_of(slot) >= total) return;
     const int K = g.K, N = g.N;
-    constexpr int EB = W8 ? 1 : 2;                        // bytes per weight element
     const int KB = K >> 7;
-    // the tile whose operands the pipeline is currently FETCHING (the next tile during a tile's last
-    // two iterations) ...
-    const uint8_t *a_ptr[NA], *b_ptr[NB];                 // this thread's chunks at k = 0
+
+    // Token rows come through a buffer descriptor and 32-bit byte offsets.  Gathered rows (row_map): one
+    // descriptor over all of x, whose size the launcher has checked against 4 GiB, so a row_map entry
+    // outside x reads zeros instead of faulting.  Sorted rows: the descriptor starts at the tile's first row.
+    const uint8_t *a_base = reinterpret_cast<const uint8_t*>(g.a), *a_base_n = a_base;
+    const int a_records = g.row_map ? (int)(uint32_t)g.a_bytes : -1;
+    uint32_t a_voff[ND], a_voff_n[ND];          // this wave's DMA offsets of the tile being fetched / of the next one
+    // bf16 weights also by DMA: descriptors of the expert's matrices and per-lane offsets
+    uint32_t b_voff[ND], b_voff_n[ND];
+    const uint8_t *bm_cur = nullptr, *bm_next = nullptr;   // matrix this wave's weight rows come from (gate or up / down)
+    // fp8 weights through registers
+    uint32_t b8_voff[NB];
+    const uint8_t *b8m0 = nullptr, *b8m1 = nullptr;
     int srow0 = 0, srow1 = 0;
     gptr_f32 sc0 = nullptr, sc1 = nullptr;
-    // ... and its output coordinates
     int row0 = 0, row_end = 0, n0 = 0;
-    int cur_e = 0;                                        // expert of the last tile looked up (tiles only move forward)
+    int cur_e = 0;
     auto setup = [&](int v) {
-    const int t = wave_s * 64 + fresh_lane();
-    const int lrow = t >> 3, lchunk = t & 7;              // bf16 tiles: row t/8 (+RA i), chunk t%8
-    const int brow = W8 ? (t >> 2) : (t >> 3);            // fp8 tiles: row t/4 (+RB i), 16-byte chunk t%4
-    const int bcol_b = W8 ? ((t & 3) << 4) : ((t & 7) << 4);   // byte offset inside the 64-element k slab
-    const int q = v / g.n_tiles_n;  // global M-tile number
-    while (uni(s_pref[cur_e + 1]) <= q) ++cur_e;        // s_pref[E] = total M tiles > q ends the walk
-    const int e = cur_e;
-    const int pe = uni(s_pref[e]);
-    const int mt_e = uni(s_pref[e + 1]) - pe;
-    int m_tile, n_tile;
-    tile_in_expert(v - pe * g.n_tiles_n, mt_e, g.n_tiles_n, m_tile, n_tile);
-    row0 = uni(s_off[e]) + m_tile * BM;
-    row_end = uni(s_off[e + 1]);
-    n0 = n_tile * NBLK;
-    // ---- per-thread load coordinates ----
+        const int l = fresh_lane();
+        const int t = wave_s * 64 + l;
+        const int q = v / g.n_tiles_n;
+        while (uni(s_pref[cur_e + 1]) <= q) ++cur_e;
+        const int e = cur_e;
+        const int pe = uni(s_pref[e]);
+        const int mt_e = uni(s_pref[e + 1]) - pe;
+        int m_tile, n_tile;
+        tile_in_expert(v - pe * g.n_tiles_n, mt_e, g.n_tiles_n, m_tile, n_tile);
+        row0 = uni(s_off[e]) + m_tile * BM;
+        row_end = uni(s_off[e + 1]);
+        n0 = n_tile * NBLK;
+        // DMA instruction i of this wave fills rows 32*wave + 8*i .. +7 of a stage: lane l supplies row +l/8 and
+        // the 16 bytes that belong at physical chunk l%8, i.e. logical chunk (l%8) ^ swz(row)
+        const int lr = l >> 3, pc = l & 7;
 #pragma unroll
-    for (int i = 0; i < NA; ++i) {
-        int r = min(row0 + lrow + RA * i, row_end - 1);
-        const int src = g.row_map ? ((gptr_i32)(uintptr_t)g.row_map)[r] : r;
-        a_ptr[i] = reinterpret_cast<const uint8_t*>(g.a + (size_t)src * K + lchunk * 8);
-    }
-    const uint8_t* bmat0 = uni_ptr(reinterpret_cast<const void*>((uintptr_t)s_ptr[0][e]));
-    const uint8_t* bmat1 = SWIGLU ? uni_ptr(reinterpret_cast<const void*>((uintptr_t)s_ptr[1][e])) : bmat0;
-    if (W8) {
-        sc0 = (gptr_f32)(uintptr_t)uni_ptr(reinterpret_cast<const void*>((uintptr_t)s_ptr[2][e]));
-        sc1 = SWIGLU ? (gptr_f32)(uintptr_t)uni_ptr(reinterpret_cast<const void*>((uintptr_t)s_ptr[3][e])) : sc0;
-    }
+        for (int i = 0; i < ND; ++i) {
+            const int rt = 32 * wave_s + 8 * i + lr;                 // row of the tile
+            const int lc = pc ^ (lr ^ (i & 1));                       // swz(rt): rt & 7 == lr, (rt >> 3) & 1 == i & 1
+            const int r = min(row0 + rt, row_end - 1);
+            const int src = g.row_map ? ((gptr_i32)(uintptr_t)g.row_map)[r] : r - row0;
+            a_voff_n[i] = (uint32_t)src * (uint32_t)(K * 2) + (uint32_t)(lc * 16);
+        }
+        if (!g.row_map) a_base_n = reinterpret_cast<const uint8_t*>(g.a) + (size_t)row0 * K * 2;
+        const uint8_t* bmat0 = uni_ptr(reinterpret_cast<const void*>((uintptr_t)s_ptr[0][e]));
+        const uint8_t* bmat1 = SWIGLU ? uni_ptr(reinterpret_cast<const void*>((uintptr_t)s_ptr[1][e])) : bmat0;
+        if (W8) {
+            sc0 = (gptr_f32)(uintptr_t)uni_ptr(reinterpret_cast<const void*>((uintptr_t)s_ptr[2][e]));
+            sc1 = SWIGLU ? (gptr_f32)(uintptr_t)uni_ptr(reinterpret_cast<const void*>((uintptr_t)s_ptr[3][e])) : sc0;
+            const int brow = t >> 2, bcol_b = (t & 3) << 4;
 #pragma unroll
-    for (int i = 0; i < NB; ++i) {
-        int r = brow + RB * i;                            // row inside the 256-row B tile
-        int n = SWIGLU ? (n0 + (r & 127)) : (n0 + r);
-        const uint8_t* m = (SWIGLU && i >= NB / 2) ? bmat1 : bmat0;  // rows >= 128 of the B tile are the up matrix
-        b_ptr[i] = m + (size_t)min(n, N - 1) * K * EB + bcol_b;
-    }
-    if (W8) {   // block-scale rows: first / second 128 rows of the B tile
-        if (SWIGLU) { srow0 = (n0 >> 7) * KB; srow1 = srow0; }
-        else        { srow0 = (n0 >> 7) * KB; srow1 = min((n0 >> 7) + 1, (N >> 7) - 1) * KB; }
-    }
-    };   // setup
-    const int lrow = tid >> 3, lchunk = tid & 7;
-    const int brow = W8 ? (tid >> 2) : (tid >> 3);
-    const uint32_t a_lds = (uint32_t)(lrow * ROW_B + ((lchunk ^ swz(lrow)) << 4));
+            for (int i = 0; i < NB; ++i) {
+                int r = brow + RB * i;
+                int n = SWIGLU ? (n0 + (r & 127)) : (n0 + r);
+                b8_voff[i] = (uint32_t)min(n, N - 1) * (uint32_t)K + (uint32_t)bcol_b;
+            }
+            b8m0 = bmat0; b8m1 = bmat1;
+            if (SWIGLU) { srow0 = (n0 >> 7) * KB; srow1 = srow0; }
+            else        { srow0 = (n0 >> 7) * KB; srow1 = min((n0 >> 7) + 1, (N >> 7) - 1) * KB; }
+        } else {
+            // rows 32*wave .. +31 of the weight tile: waves 0-3 the first 128 rows (gate), 4-7 the second (up)
+            bm_next = (SWIGLU && wave_s >= 4) ? bmat1 : bmat0;
+#pragma unroll
+            for (int i = 0; i < ND; ++i) {
+                const int rt = 32 * wave_s + 8 * i + lr;
+                const int lc = pc ^ (lr ^ (i & 1));
+                const int n = SWIGLU ? (n0 + (rt & 127)) : (n0 + rt);
+                b_voff_n[i] = (uint32_t)min(n, N - 1) * (uint32_t)(K * 2) + (uint32_t)(lc * 16);
+            }
+        }
+    };
+    auto adopt = [&]() {   // the next tile's DMA coordinates become the current ones
+#pragma unroll
+        for (int i = 0; i < ND; ++i) { a_voff[i] = a_voff_n[i]; if (!W8) b_voff[i] = b_voff_n[i]; }
+        if (!W8) bm_cur = bm_next;
+        a_base = a_base_n;
+    };
+    auto dma_a = [&](uint8_t* stA, int kt, int i) {
+        const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)a_base, 0, a_records, 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lds_u8)(stA + (32 * wave_s + 8 * i) * ROW_B), 16, a_voff[i],
+                                                 (uint32_t)(kt * BK * 2), 0, 0);
+    };
+    auto dma_b = [&](uint8_t* stB, int kt, int i) {
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)bm_cur, 0, -1, 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_u8)(stB + (32 * wave_s + 8 * i) * ROW_B), 16, b_voff[i],
+                                                 (uint32_t)(kt * BK * 2), 0, 0);
+    };
+    // fp8 weight path (registers): thread t owns row t/4 (+128 i), chunks 2q, 2q+1 of the bf16 row
+    const int brow = tid >> 2;
     uint32_t b_lds[2];
-    // fp8: a thread owns chunks 2q and 2q+1 of its row; rows with bit 1 set store them in the
-    // opposite order so that the 16 lanes of one store instruction (4 rows x 4 chunks) spread
-    // over all banks
     const bool b_swap = W8 && ((brow >> 1) & 1);
-    if (W8) {
+    {
         int qd = tid & 3, sw = swz(brow), first = b_swap ? 1 : 0;
         b_lds[0] = (uint32_t)(brow * ROW_B + (((2 * qd + first) ^ sw) << 4));
         b_lds[1] = (uint32_t)(brow * ROW_B + (((2 * qd + 1 - first) ^ sw) << 4));
-    } else {
-        b_lds[0] = (uint32_t)(brow * ROW_B + (((tid & 7) ^ swz(brow)) << 4));
-        b_lds[1] = 0;
     }
-
-    // PF register sets: global loads run PF tiles ahead of the LDS stores.  One set when the
-    // workgroup is compute bound (BM = 256, which has no registers to spare); two for the smaller
-    // tiles, which mostly stream weights (decode) and where bytes in flight per CU are what
-    // limits the HBM rate.
-    constexpr int PF = (MT <= 2) ? 2 : 1;
-    u32x4 ra[PF][NA], rb[PF][NB];
-    float rs[PF][2];
-    auto gload = [&](int kt, int set) {
+    u32x4 rb[NB];
+    float rs[2];
+    auto load_b8 = [&](int i, uint32_t kofs) {
+        const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)((SWIGLU && i >= NB / 2) ? b8m1 : b8m0), 0, -1, 0x00020000);
+        return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, b8_voff[i], kofs, 0));
+    };
+    auto gload_b = [&](int kt) {
         const size_t kofs = (size_t)kt * BK;
 #pragma unroll
-        for (int i = 0; i < NA; ++i) ra[set][i] = gload16(a_ptr[i] + kofs * 2);
+        for (int i = 0; i < NB; ++i) rb[i] = load_b8(i, (uint32_t)kofs);
+        rs[0] = sc0[srow0 + (kt >> 1)];
+        rs[1] = sc1[srow1 + (kt >> 1)];
+    };
+    auto store_b_all = [&](uint8_t* Bs) {
 #pragma unroll
-        for (int i = 0; i < NB; ++i) rb[set][i] = gload16(b_ptr[i] + kofs * EB);
-        if (W8) {
-            rs[set][0] = sc0[srow0 + (kt >> 1)];
-            rs[set][1] = sc1[srow1 + (kt >> 1)];
+        for (int i = 0; i < NB; ++i) {
+            u32x4 l, h;
+            dequant16(rb[i], rs[i / (NB / 2)], l, h);
+            *reinterpret_cast<u32x4*>(Bs + b_lds[0] + i * RB * ROW_B) = b_swap ? h : l;
+            *reinterpret_cast<u32x4*>(Bs + b_lds[1] + i * RB * ROW_B) = b_swap ? l : h;
         }
     };
-    auto lds_store = [&](uint8_t* As, int set) {
-        uint8_t* Bs = As + A_STAGE;
-#pragma unroll
-        for (int i = 0; i < NA; ++i) *reinterpret_cast<u32x4*>(As + a_lds + i * RA * ROW_B) = ra[set][i];
-        if (W8) {
-#pragma unroll
-            for (int i = 0; i < NB; ++i) {
-                u32x4 l, h;
-                dequant16(rb[set][i], rs[set][i / (NB / 2)], l, h);
-                *reinterpret_cast<u32x4*>(Bs + b_lds[0] + i * RB * ROW_B) = b_swap ? h : l;
-                *reinterpret_cast<u32x4*>(Bs + b_lds[1] + i * RB * ROW_B) = b_swap ? l : h;
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < NB; ++i) *reinterpret_cast<u32x4*>(Bs + b_lds[0] + i * RB * ROW_B) = rb[set][i];
+    auto b_item = [&](int it, uint8_t* Bs, int kn) {   // it in 0 .. 2*NB-1: half it%2 of chunk it/2
+        const int b = it >> 1, half = it & 1;
+        const u32x4 o = dequant8(rb[b][2 * half], rb[b][2 * half + 1], rs[b / (NB / 2)]);
+        *reinterpret_cast<u32x4*>(Bs + ((half ^ (b_swap ? 1 : 0)) ? b_lds[1] : b_lds[0]) + b * RB * ROW_B) = o;
+        if (half == 1) {
+            rb[b] = load_b8(b, (uint32_t)(kn * BK));
+            if (b / (NB / 2) == 0) rs[0] = sc0[srow0 + (kn >> 1)];
+            else rs[1] = sc1[srow1 + (kn >> 1)];
         }
     };
 
-    // ---- MFMA operand coordinates (v_mfma_f32_16x16x32_bf16) ----
-    // fragment row = base + lane%16 (bases are multiples of 16); logical chunk = 4*s + lane/16 for
-    // the 32-wide k-step s of the stage: lane l supplies k = 8*(l/16) .. +7 of row l%16
     const int frow = lane & 15, fquad = lane >> 4, fkey = swz(frow);
-    // The LDS serves a 16-byte read 8 + 8 lanes at a time (lanes 8i.. together with 32+8i..):
-    // such a pair of lane groups must read neighbouring chunks of the same rows, which is what the
-    // swizzle keeps conflict-free, so lane group q takes chunk 0,2,1,3 of the k-step instead of q
-    // (with q the counter SQ_LDS_BANK_CONFLICT reads 22 % of the busy cycles, with this order
-    // 0.3 %).  Both operands use the same order, and a dot product does not care in which order
-    // k is walked.
     const int fchunk = ((fquad & 1) << 1) | (fquad >> 1);
-    constexpr int TM = 2 * MT, TN = 2 * NJ;       // 16-row token tiles / 16-row weight tiles per wave
+    constexpr int TM = 2 * MT, TN = 2 * NJ;
     uint32_t tok_off[TM], w_off[TN];
 #pragma unroll
     for (int mi = 0; mi < TM; ++mi) tok_off[mi] = (uint32_t)((wm * 32 * MT + 16 * mi + frow) * ROW_B);
@@ -748,24 +773,12 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
         int r = SWIGLU ? ((j < TN / 2 ? 0 : 128) + wn * (8 * TN) + 16 * (j % (TN / 2))) : (wn * (16 * TN) + 16 * j);
         w_off[j] = (uint32_t)((r + frow) * ROW_B);
     }
-
     f32x4 acc[TM][TN];
-#pragma unroll
-    for (int mi = 0; mi < TM; ++mi)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[mi][j] = f32x4{0};
-
-    // A stage is multiplied in NU sub-phases: k-step s (32 wide) x token part q (TQ tiles), each
-    // TQ x TN MFMAs.  Weight fragments are double-buffered by k-step; token parts ping-pong between
-    // two small buffers.  Slot v of an iteration issues the MFMAs of sub-phase v-2 (the last two
-    // sub-phases of a stage run in the first two slots of the next iteration, across the workgroup
-    // barrier) and then requests the fragments of sub-phase v, whose buffer those MFMAs just freed.
-    constexpr int TQ = (MT >= 2) ? MT / 2 : 1;    // token tiles per part
-    constexpr int NP = TM / TQ;                   // parts per k-step
-    constexpr int NU = 2 * NP;                    // sub-phases per stage
+    constexpr int TQ = MT / 2;
+    constexpr int NP = TM / TQ;
+    constexpr int NU = 2 * NP;
     bf16x8 wfr[2][TN], tq[2][TQ];
-    auto read_w1 = [&](const uint8_t* As, int s, int j) {
-        const uint8_t* Bs = As + A_STAGE;
+    auto read_w1 = [&](const uint8_t* Bs, int s, int j) {
         const uint32_t coff = (uint32_t)(((4 * s + fchunk) ^ fkey) << 4);
         wfr[s][j] = *reinterpret_cast<const bf16x8*>(Bs + w_off[j] + coff);
     };
@@ -781,143 +794,89 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
         for (int i = 0; i < TQ; ++i)
 #pragma unroll
             for (int jx = 0; jx < TN; ++jx) {
-                // snake order over the weight fragments: every instruction differs from the one before in
-                // ONE operand (fewer input toggles per MFMA on a power-limited chip; +0.4 % measured)
                 const int j = ((i + u) & 1) ? TN - 1 - jx : jx;
                 acc[q * TQ + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wfr[s][j], tq[u & 1][i], acc[q * TQ + i][j], 0, 0, 0);
             }
     };
-    // ---- main loop ----
-    // On entry to iteration kt: LDS stage kt&1 holds tile kt and the registers hold tiles kt+1 ..
-    // kt+PF (possibly still in flight).  The iteration moves tile kt+1 into the other LDS stage,
-    // refills that register set with tile kt+1+PF and multiplies tile kt.
     const int nk = K / BK;
-    // One data item = one LDS store's worth of this thread's staged chunks (a 16-byte token chunk,
-    // a 16-byte bf16 weight chunk, or half of a 16-byte fp8 weight chunk -> 8 bf16): store it to the
-    // other stage and, once a chunk's last item is stored, refill its registers with the chunk of
-    // tile kt+1+PF.  The items are spread over the iteration, one per group of MFMAs, so LDS, the
-    // vector-memory pipe and the matrix core see a steady mix instead of bursts; with exact load
-    // waits each item stalls only until its own chunk (requested PF iterations earlier) is there.
-    constexpr int NBI = W8 ? 2 * NB : NB;
-    constexpr int NI = NA + NBI;
-    auto data_item = [&](int i, uint8_t* As, int kn, int set) {   // kn: k-stage (of the tile being fetched) to request
-        uint8_t* Bs = As + A_STAGE;
-        const size_t kofs = (size_t)kn * BK;
-        if (i < NA) {
-            *reinterpret_cast<u32x4*>(As + a_lds + i * RA * ROW_B) = ra[set][i];
-            ra[set][i] = gload16(a_ptr[i] + kofs * 2);
-        } else if (W8) {
-            const int b = (i - NA) >> 1, half = (i - NA) & 1;
-            const float sc = rs[set][b / (NB / 2)];
-            const u32x4 o = dequant8(rb[set][b][2 * half], rb[set][b][2 * half + 1], sc);
-            // the first 8 weights go to b_lds[0], the second 8 to b_lds[1]; swapped rows the other way round
-            *reinterpret_cast<u32x4*>(Bs + ((half ^ (b_swap ? 1 : 0)) ? b_lds[1] : b_lds[0]) + b * RB * ROW_B) = o;
-            if (half == 1) {
-                rb[set][b] = gload16(b_ptr[b] + kofs * EB);
-                if (b / (NB / 2) == 0) rs[set][0] = sc0[srow0 + (kn >> 1)];
-                else rs[set][1] = sc1[srow1 + (kn >> 1)];
-            }
-        } else {
-            const int b = i - NA;
-            *reinterpret_cast<u32x4*>(Bs + b_lds[0] + b * RB * ROW_B) = rb[set][b];
-            rb[set][b] = gload16(b_ptr[b] + kofs * EB);
-        }
-    };
-    constexpr int NG = NU;                        // one group of MFMAs per slot
-    constexpr int WPS = TN / NP;                  // weight fragments of the second k-step read per slot
-    auto iteration = [&](int kt, int kn, int set, int par) {   // par == kt & 1
-        const uint8_t* rd = par ? smem1 : smem0;
-        uint8_t* wr = par ? smem0 : smem1;
+    constexpr int WPS = TN / NP;
+    // iteration kt multiplies stage par; the DMA brings k-stage ka (of the tile whose coordinates are current) into
+    // the other token stage (and weight stage, bf16); fp8 converts the weight registers (k-stage kt+1) into the other
+    // weight stage and refills them with k-stage kb
+    auto iteration = [&](int kt, int ka, int kb, int par) {
+        const uint8_t* rdA = par ? sA1 : sA0; const uint8_t* rdB = par ? sB1 : sB0;
+        uint8_t* wrA = par ? sA0 : sA1; uint8_t* wrB = par ? sB0 : sB1;
 #pragma unroll
         for (int v = 0; v < NU; ++v) {
-            // group v takes items [v*NI/NG, (v+1)*NI/NG): in order, so the two halves of an fp8
-            // chunk are stored before its registers are refilled
-#pragma unroll
-            for (int i0 = v * NI / NG; i0 < (v + 1) * NI / NG; ++i0) {
-                const int i = (W8 && NA == 4 && NI == 8) ? ((i0 & 1) ? NA + (i0 >> 1) : (i0 >> 1)) : i0;
-                data_item(i, wr, kn, set);
+            if (v < ND) {
+                dma_a(wrA, ka, v);
+                if (!W8) dma_b(wrB, ka, v);
+            } else if (W8) {
+                b_item(v - ND, wrB, kb);
             }
             if (!W8) __builtin_amdgcn_sched_barrier(0);
             if (v >= 2) mfma_sub(v - 2);
             else if (kt > 0) mfma_sub(NU - 2 + v);
-            read_tq(rd, v);
+            read_tq(rdA, v);
             if (v == 0) {
 #pragma unroll
-                for (int j = 0; j < TN; ++j) read_w1(rd, 0, j);
+                for (int j = 0; j < TN; ++j) read_w1(rdB, 0, j);
             } else if (v >= 2 && v < 2 + NP) {
 #pragma unroll
-                for (int j = (v - 2) * WPS; j < (v - 1) * WPS; ++j) read_w1(rd, 1, j);
+                for (int j = (v - 2) * WPS; j < (v - 1) * WPS; ++j) read_w1(rdB, 1, j);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        __syncthreads();   // (waits for this wave's LDS reads and writes, then for the other waves)
+        // this wave's DMA has landed (the four younger loads are the fp8 weight chunks and scales), then everybody's
+        if (W8) asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
     };
+    static_assert(NU == 8 && ND == 4 && (!W8 || NB == 2), "slot plan");
     // ---- tiles ----
-    static_assert(PF == 1, "the tile hand-over below assumes one register set");
     setup(tile_of(slot));
-    gload(0, 0);
-    lds_store(smem0, 0);
-    gload(1, 0);
+    adopt();
+#pragma unroll
+    for (int i = 0; i < ND; ++i) { dma_a(sA0, 0, i); if (!W8) dma_b(sB0, 0, i); }
+    if (W8) {
+        gload_b(0);
+        store_b_all(sB0);
+        gload_b(1);
+        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
     __syncthreads();
-    constexpr int CW = SWIGLU ? 8 * TN : 16 * TN;    // output columns of this wave
-    constexpr int RBW = CW * 2;                      // bytes per output row of this wave
-    constexpr int CPR = RBW / 16;                    // 16-byte chunks per row (4 or 8)
-    constexpr int KSH = CPR == 8 ? 0 : 1;            // swizzle key = (row >> KSH) & (CPR-1)
-    constexpr int RPP = 64 / CPR;                    // rows per read-back pass
+    constexpr int CW = SWIGLU ? 8 * TN : 16 * TN;
+    constexpr int RBW = CW * 2;
+    constexpr int CPR = RBW / 16;
+    constexpr int KSH = CPR == 8 ? 0 : 1;
+    constexpr int RPP = 64 / CPR;
     for (;;) {
         const int out_row0 = row0, out_row_end = row_end, out_n0 = n0;
 #pragma unroll
         for (int mi = 0; mi < TM; ++mi)
 #pragma unroll
             for (int j = 0; j < TN; ++j) acc[mi][j] = f32x4{0};
-        // k-iterations 0 .. nk-3 fetch this tile's stages 2 .. nk-1 (nk is even and >= 2); the last two
-        // fetch stages 0 and 1 of the next tile, whose coordinates are looked up right before them
-        // (no tile left: this tile's last stage again, stored where nobody reads it).
         bool more = false;
-        if (W8) {
-            // fp8: the k loop is unrolled by two with literal stage parities, and the two hand-over
-            // iterations are a copy of their own behind it (folded into the loop body the kernel
-            // needs no spill at all, but the gate/up shape measured 3 % slower)
-            for (int kt = 0; kt + 2 <= nk - 2; kt += 2) {
-                iteration(kt, kt + 2, 0, 0);
-                iteration(kt + 1, kt + 3, 0, 1);
-            }
-            slot += slots;
-            more = tile_of(slot) < total;
-            setup(tile_of(more ? slot : slot - slots));
-            iteration(nk - 2, more ? 0 : nk - 1, 0, 0);
-            iteration(nk - 1, more ? 1 : nk - 1, 0, 1);
-        } else {
-            // bf16 (4 instead of 2 weight chunks in flight per thread) has no registers for a second
-            // copy of the iteration: one rolled loop, the lookup under a uniform branch in front of
-            // the hand-over iterations (a copy of its own spills 30-46 registers, and every reload is a
-            // vmcnt(0) that drains the prefetch)
-            for (int kt = 0; kt < nk; ++kt) {
-                if (kt == nk - 2) {
-                    slot += slots;
-                    more = tile_of(slot) < total;
-                    setup(tile_of(more ? slot : slot - slots));
-                }
-                const int kn = kt + 2 < nk ? kt + 2 : (more ? kt + 2 - nk : nk - 1);
-                iteration(kt, kn, 0, kt & 1);
-            }
+        for (int kt = 0; kt + 2 <= nk - 2; kt += 2) {
+            iteration(kt, kt + 1, kt + 2, 0);
+            iteration(kt + 1, kt + 2, kt + 3, 1);
         }
+        slot += slots;
+        more = tile_of(slot) < total;
+        setup(tile_of(more ? slot : slot - slots));
+        iteration(nk - 2, nk - 1, more ? 0 : nk - 1, 0);
+        adopt();
+        iteration(nk - 1, more ? 0 : nk - 1, more ? 1 : nk - 1, 1);
         mfma_sub(NU - 2);
         mfma_sub(NU - 1);
 
-        // ---- epilogue ----
-        // acc[mi][j][i]: token row = 16*mi + lane%16 of the wave's M range; output column
-        // = 16*j + 4*(lane/16) + i of the wave's N range, i.e. a lane holds 4 consecutive columns
-        // (8 bytes) of one row per accumulator.  Stage 0 already holds the next tile; stage 1 is idle
-        // until the next tile's first iteration writes it, so each wave transposes its outputs through
-        // its 8 KiB slice of stage 1 (64 or 128 rows at a time) and writes 16 bytes per lane, whole
-        // 64/128-byte row segments per 4/8 lanes.
-        const int rows_here = min(BM, out_row_end - out_row0) - wm * 32 * MT;   // valid rows of this wave
+        const int rows_here = min(BM, out_row_end - out_row0) - wm * 32 * MT;
         const int ncol0 = out_n0 + wn * CW;
         const int el = fresh_lane();
         const int efrow = el & 15, efquad = el >> 4, rr = el / CPR, cc = el % CPR;
-        uint8_t* ep = smem1 + wave_s * 8192;
-        constexpr int RPW = 8192 / RBW;                  // rows per pass (128 or 64)
+        uint8_t* ep = ((wave_s < 4) ? sA1 : sB1) + (wave_s & 3) * 8192;
+        constexpr int RPW = 8192 / RBW;
 #pragma unroll
         for (int pass = 0; pass < 32 * MT / RPW; ++pass) {
 #pragma unroll
@@ -939,18 +898,14 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
                 if (pass * RPW + r < rows_here && ncol0 + cc * 8 < N)
                 {
                     u32x4* dst = reinterpret_cast<u32x4*>(g.c + (size_t)(out_row0 + wm * 32 * MT + pass * RPW + r) * N + ncol0 + cc * 8);
-                    // down projection: whole 128-byte lines per 8 lanes, written non-temporally (the
-                    // pipeline's next load waits also cover these stores; -0.8 %).  The gate/up
-                    // launch writes half lines per wave: plain stores, so that L2 merges the halves.
                     if (SWIGLU) *dst = v; else __builtin_nontemporal_store(v, dst);
                 }
             }
         }
         if (!more) return;
-        __syncthreads();   // every wave has read its outputs back: the next tile may write stage 1
+        __syncthreads();
     }
 }
-
 
 template <int MT, int WN, bool SWIGLU, bool W8>
 int launch_one(const GemmArgs& g, int n_rows, hipStream_t st) {
@@ -995,8 +950,9 @@ template <bool SWIGLU, bool W8>
 int launch_mt(const GemmArgs& g, int n_rows, hipStream_t st) {
     const long mean = g.E > 0 ? (long)n_rows / g.E : 0;
     // the persistent kernel needs an even number of k-stages for its hand-over (fp8 sizes always have
-    // one) and keeps per-expert tables for up to 512 experts
-    if (mean >= 192 && g.K % 128 == 0 && g.E <= 512 && cu_count() >= 8) return launch_persistent<SWIGLU, W8>(g, n_rows, st);
+    // one), keeps per-expert tables for up to 512 experts and addresses gathered rows with 32-bit offsets
+    const bool fits = !g.row_map || g.a_bytes < (1ull << 32);
+    if (mean >= 192 && g.K % 128 == 0 && g.E <= 512 && fits && cu_count() >= 8) return launch_persistent<SWIGLU, W8>(g, n_rows, st);
     // The counts themselves live on the device; only their mean is known here.  Routing is
     // uneven, so around a mean of 64 rows some experts exceed 64 and would stream their weights
     // once per 64-row tile: 128-row tiles from a mean of 48 (Mixtral-8x22B decode, 256 tokens:
@@ -1007,7 +963,7 @@ int launch_mt(const GemmArgs& g, int n_rows, hipStream_t st) {
 }
 
 template <bool W8>
-int grouped_swiglu(const void* x, const int32_t* row_map, const void* const* w_gate, const void* const* w_up,
+int grouped_swiglu(const void* x, int32_t x_rows, const int32_t* row_map, const void* const* w_gate, const void* const* w_up,
                    const void* const* w_down, const float* const* s_gate, const float* const* s_up,
                    const float* const* s_down, const int32_t* offsets, int32_t n_rows, int32_t n_experts,
                    int32_t hidden, int32_t inter, void* act, void* y, int32_t phases, void* stream, const char* who) {
@@ -1015,6 +971,7 @@ int grouped_swiglu(const void* x, const int32_t* row_map, const void* const* w_g
     MOE_REQUIRE(phases >= MOE_PHASE_GATE_UP && phases <= MOE_PHASE_BOTH, "%s: bad phases %d", who, phases);
     if (n_rows == 0) return MOE_OK;
     MOE_REQUIRE(x && w_gate && w_up && w_down && offsets && act && y, "%s: NULL pointer argument", who);
+    MOE_REQUIRE(x_rows >= 1, "%s: x_rows %d < 1", who, x_rows);
     MOE_REQUIRE(!W8 || (s_gate && s_up && s_down), "%s: NULL scale pointer array", who);
     MOE_REQUIRE(n_experts >= 1 && n_experts <= MAX_E, "%s: n_experts %d outside [1,%d]", who, n_experts, MAX_E);
     const int align = W8 ? 128 : 64;
@@ -1025,6 +982,7 @@ int grouped_swiglu(const void* x, const int32_t* row_map, const void* const* w_g
     GemmArgs g1{};
     g1.a = static_cast<const uint16_t*>(x);
     g1.row_map = row_map;
+    g1.a_bytes = (size_t)x_rows * (size_t)hidden * 2;
     g1.b0 = w_gate; g1.b1 = w_up; g1.s0 = s_gate; g1.s1 = s_up;
     g1.offsets = offsets;
     g1.c = static_cast<uint16_t*>(act);
@@ -1074,21 +1032,21 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
 
 extern "C" size_t moe_grouped_workspace_bytes(int32_t, int32_t) { return 256; }
 
-extern "C" int moe_grouped_swiglu_bf16(const void* x, const int32_t* row_map, const void* const* w_gate,
+extern "C" int moe_grouped_swiglu_bf16(const void* x, int32_t x_rows, const int32_t* row_map, const void* const* w_gate,
                                        const void* const* w_up, const void* const* w_down, const int32_t* offsets,
                                        int32_t n_rows, int32_t n_experts, int32_t hidden, int32_t inter, void* act,
                                        void* y, int32_t phases, void*, size_t, void* stream) {
-    return moe::grouped_swiglu<false>(x, row_map, w_gate, w_up, w_down, nullptr, nullptr, nullptr, offsets, n_rows,
+    return moe::grouped_swiglu<false>(x, x_rows, row_map, w_gate, w_up, w_down, nullptr, nullptr, nullptr, offsets, n_rows,
                                       n_experts, hidden, inter, act, y, phases, stream, "moe_grouped_swiglu_bf16");
 }
 
-extern "C" int moe_grouped_swiglu_w8a16(const void* x, const int32_t* row_map, const void* const* w_gate,
+extern "C" int moe_grouped_swiglu_w8a16(const void* x, int32_t x_rows, const int32_t* row_map, const void* const* w_gate,
                                         const void* const* w_up, const void* const* w_down,
                                         const float* const* s_gate, const float* const* s_up,
                                         const float* const* s_down, const int32_t* offsets, int32_t n_rows,
                                         int32_t n_experts, int32_t hidden, int32_t inter, void* act, void* y,
                                         int32_t phases, void*, size_t, void* stream) {
-    return moe::grouped_swiglu<true>(x, row_map, w_gate, w_up, w_down, s_gate, s_up, s_down, offsets, n_rows,
+    return moe::grouped_swiglu<true>(x, x_rows, row_map, w_gate, w_up, w_down, s_gate, s_up, s_down, offsets, n_rows,
                                      n_experts, hidden, inter, act, y, phases, stream, "moe_grouped_swiglu_w8a16");
 }
 

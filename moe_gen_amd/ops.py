@@ -208,12 +208,12 @@ def grouped_swiglu(x: torch.Tensor, row_map, ptrs: ExpertPointers, offsets: torc
             raise ValueError(f"rows_bound {rows_bound} outside [0, {n_rows}]")
         n_rows = rows_bound
     if ptrs.fp8:
-        N.check(L.moe_grouped_swiglu_w8a16(_ptr(x), _ptr(row_map), _ptr(ptrs.w_gate), _ptr(ptrs.w_up),
+        N.check(L.moe_grouped_swiglu_w8a16(_ptr(x), x.shape[0], _ptr(row_map), _ptr(ptrs.w_gate), _ptr(ptrs.w_up),
                                            _ptr(ptrs.w_down), _ptr(ptrs.s_gate), _ptr(ptrs.s_up),
                                            _ptr(ptrs.s_down), _ptr(offsets), n_rows, E, h, I, _ptr(act), _ptr(y),
                                            phases, None, 0, _stream()), "moe_grouped_swiglu_w8a16")
     else:
-        N.check(L.moe_grouped_swiglu_bf16(_ptr(x), _ptr(row_map), _ptr(ptrs.w_gate), _ptr(ptrs.w_up),
+        N.check(L.moe_grouped_swiglu_bf16(_ptr(x), x.shape[0], _ptr(row_map), _ptr(ptrs.w_gate), _ptr(ptrs.w_up),
                                           _ptr(ptrs.w_down), _ptr(offsets), n_rows, E, h, I, _ptr(act), _ptr(y),
                                           phases, None, 0, _stream()), "moe_grouped_swiglu_bf16")
     return y

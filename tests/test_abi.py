@@ -49,6 +49,6 @@ def test_argument_validation_needs_no_gpu():
     assert lib.moe_router(1, 1, None, ctypes.byref(p), 1, 1, None, None) == -1
     assert "scoring" in N.last_error()
     assert lib.moe_combine(1, 1, None, 1, None, 4, 99, 64, 0, 1, None) == -1 and "top_k" in N.last_error()
-    assert lib.moe_grouped_swiglu_bf16(1, None, 1, 1, 1, 1, 8, 2, 100, 64, 1, 1, 3, None, 0, None) == -1
+    assert lib.moe_grouped_swiglu_bf16(1, 8, None, 1, 1, 1, 1, 8, 2, 100, 64, 1, 1, 3, None, 0, None) == -1
     assert "hidden" in N.last_error()
     assert lib.moe_dispatch(1, 4, 2, 300, 1, 1, 1, 1, None, None, 0, None, None, 0, None) == -1

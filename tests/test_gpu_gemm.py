@@ -149,6 +149,93 @@ def test_grouped_swiglu_row_map(fp8):
     assert rel_max(y, ref32) <= TOL
 
 
+def _one_expert(h, I, seed):
+    from moe_gen_amd import ops
+    g = torch.Generator().manual_seed(seed)
+    ws = [(torch.randn(shape, generator=g) * 0.05).to(torch.bfloat16) for shape in ((I, h), (I, h), (h, I))]
+    ptrs = ops.expert_pointers(*[[w.cuda()] for w in ws])
+    return ws, ptrs
+
+
+def test_row_map_entry_outside_x_reads_zeros():
+    """The persistent kernel fetches gathered rows through a buffer descriptor that ends with x: a
+    row_map entry beyond x_rows reads a row of zeros (no fault), and every other row is unaffected."""
+    from moe_gen_amd import ops
+    h, I, n = 256, 256, 600
+    ws, ptrs = _one_expert(h, I, 41)
+    g = torch.Generator().manual_seed(42)
+    x = torch.randn(n, h, generator=g).to(torch.bfloat16)
+    rm = torch.randperm(n, generator=g).to(torch.int32)
+    bad = [3, 257, 599]
+    rm_bad = rm.clone()
+    rm_bad[bad] = torch.tensor([n, n + 5, 2 ** 20], dtype=torch.int32)
+    off = torch.tensor([0, n], dtype=torch.int32, device="cuda")
+    y_ok = ops.grouped_swiglu(x.cuda(), rm.cuda(), ptrs, off, n)
+    y_bad = ops.grouped_swiglu(x.cuda(), rm_bad.cuda(), ptrs, off, n)
+    torch.cuda.synchronize()
+    keep = np.ones(n, bool)
+    keep[bad] = False
+    assert np.array_equal(bits(y_ok)[keep], bits(y_bad)[keep])
+    assert (y_bad[bad].float().cpu().numpy() == 0).all()        # silu(0) * 0 through the down projection
+
+
+def test_gathered_rows_of_an_input_beyond_4_gib():
+    """Gathered rows are addressed with 32-bit byte offsets only while x is smaller than 4 GiB; a larger
+    x takes the one-workgroup-per-tile kernel with 64-bit addresses.  The rows used sit at both ends of x."""
+    from moe_gen_amd import ops
+    h, I, n = 2048, 256, 512
+    x_rows = (1 << 32) // (h * 2) + 4096                          # 4 GiB + 16 MiB of bf16 rows
+    ws, ptrs = _one_expert(h, I, 43)
+    g = torch.Generator().manual_seed(44)
+    rows = torch.randn(n, h, generator=g).to(torch.bfloat16)
+    x = torch.zeros(x_rows, h, dtype=torch.bfloat16, device="cuda")
+    where = torch.cat([torch.arange(n // 2), torch.arange(x_rows - n // 2, x_rows)]).to(torch.int32)
+    where = where[torch.randperm(n, generator=g)]
+    x[where.long().cuda()] = rows.cuda()
+    off = torch.tensor([0, n], dtype=torch.int32, device="cuda")
+    y = ops.grouped_swiglu(x, where.cuda(), ptrs, off, n)
+    y_ref = ops.grouped_swiglu(rows.cuda(), None, ptrs, off, n)   # the same rows, sorted: the persistent kernel
+    torch.cuda.synchronize()
+    del x
+    wg, wu, wd = (O.bf16_to_f32(bits(w)) for w in ws)
+    ref32 = O.mlp_f32(O.bf16_to_f32(bits(rows)), wg, wu, wd)
+    assert rel_max(O.bf16_to_f32(bits(y)), ref32) <= TOL
+    assert rel_max(O.bf16_to_f32(bits(y_ref)), ref32) <= TOL
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_expert_sub_range_through_the_persistent_kernel(fp8):
+    """A call on experts [1, 3) of four with absolute row offsets (weights handed out in waves): the rows
+    of the other experts stay untouched, the range's rows match the call on all experts."""
+    from moe_gen_amd import ops
+    E, h, I = 4, 256, 256
+    counts = np.array([300, 520, 260, 290], np.int32)
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    n = int(offsets[-1])
+    g = torch.Generator().manual_seed(47)
+    x = torch.randn(n, h, generator=g).to(torch.bfloat16).cuda()
+    mats = make_experts(E, h, I, fp8, 48)
+    dev = lambda m: tuple(t.cuda() for t in m) if isinstance(m, tuple) else m.cuda()
+    dm = [[dev(m) for m in one] for one in mats]
+
+    def pointers(sel):
+        if fp8:
+            return ops.expert_pointers([dm[e][0][0] for e in sel], [dm[e][1][0] for e in sel], [dm[e][2][0] for e in sel],
+                                       [dm[e][0][1] for e in sel], [dm[e][1][1] for e in sel], [dm[e][2][1] for e in sel])
+        return ops.expert_pointers([dm[e][0] for e in sel], [dm[e][1] for e in sel], [dm[e][2] for e in sel])
+
+    off_d = torch.from_numpy(offsets).cuda()
+    y_all = ops.grouped_swiglu(x, None, pointers(range(E)), off_d, n)
+    act = torch.zeros(n, I, dtype=torch.bfloat16, device="cuda")
+    y = torch.full((n, h), 7.0, dtype=torch.bfloat16, device="cuda")
+    ops.grouped_swiglu(x, None, pointers([1, 2]), off_d[1:4].contiguous(), n, act, y,
+                       rows_bound=int(offsets[3] - offsets[1]))
+    torch.cuda.synchronize()
+    a, b = int(offsets[1]), int(offsets[3])
+    assert torch.equal(y[a:b], y_all[a:b])
+    assert (y[:a] == 7.0).all() and (y[b:] == 7.0).all()
+
+
 def test_grouped_single_expert_is_plain_mlp():
     """E = 1 reduces to a dense SwiGLU MLP: compare with torch's own bf16 linear layers on the GPU."""
     from moe_gen_amd import DeepseekV3Config, DeepseekV3MLP
