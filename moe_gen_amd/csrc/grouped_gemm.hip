@@ -158,6 +158,106 @@ __device__ __forceinline__ u32x2 epilogue_pack(const f32x4& a, const f32x4& up) 
     return u32x2{pack_bf16(a[0], a[1]), pack_bf16(a[2], a[3])};
 }
 
+// Exclusive scan of the experts' M-tile counts, ceil(count / BM), by the whole workgroup: s_pref[e] = number of
+// M tiles in front of expert e (the caller adds s_pref[E] if it needs it).  Returns the total; the thread that
+// handled expert tid in the LAST pass keeps that expert's prefix, tile count and row range in `mine`
+// (experts beyond NT take further passes), and per_expert(e, first_row, end_row) runs once per expert.
+struct ExpertOfThread { int start, mt, o0, o1; };
+template <int NT, int BM, typename F>
+__device__ __forceinline__ int mtile_prefix_scan(const GemmArgs& g, int tid, int* s_pref, int* s_wtot,
+                                                 ExpertOfThread& mine, F per_expert) {
+    const int lane = tid & 63, wave = tid >> 6;
+    int run = 0;
+    mine = ExpertOfThread{0, 0, 0, 0};
+    for (int e0 = 0; e0 < g.E; e0 += NT) {
+        const int e = e0 + tid;
+        int mt = 0;
+        if (e < g.E) {
+            mine.o0 = g.offsets[e];
+            mine.o1 = g.offsets[e + 1];
+            mt = (mine.o1 - mine.o0 + BM - 1) / BM;
+            per_expert(e, mine.o0, mine.o1);
+        }
+        int inc = mt;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            int o = __shfl_up(inc, d);
+            if (lane >= d) inc += o;
+        }
+        if (lane == 63) s_wtot[wave] = inc;
+        __syncthreads();
+        int pre = run, tot = 0;
+#pragma unroll
+        for (int w = 0; w < NT / 64; ++w) {
+            if (w < wave) pre += s_wtot[w];
+            tot += s_wtot[w];
+        }
+        mine.start = pre + inc - mt;
+        mine.mt = mt;
+        if (e < g.E) s_pref[e] = mine.start;
+        run += tot;
+        if (g.E > NT) __syncthreads();   // s_wtot is rewritten by the next pass
+    }
+    return run;
+}
+
+// LDS row offsets of a wave's MFMA operand fragments (v_mfma_f32_16x16x32_bf16): fragment row = base + lane%16,
+// bases multiples of 16.  Tokens: the wave's 32*MT rows; weights: TN fragments of 16 rows, for SWIGLU the first
+// half from the gate rows (0..127 of the tile) and the second half from the matching up rows (128..255).
+template <int MT, int TN, bool SWIGLU>
+__device__ __forceinline__ void fragment_rows(int wm, int wn, int frow, uint32_t (&tok_off)[2 * MT], uint32_t (&w_off)[TN]) {
+#pragma unroll
+    for (int mi = 0; mi < 2 * MT; ++mi) tok_off[mi] = (uint32_t)((wm * 32 * MT + 16 * mi + frow) * ROW_B);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int r = SWIGLU ? ((j < TN / 2 ? 0 : 128) + wn * (8 * TN) + 16 * (j % (TN / 2))) : (wn * (16 * TN) + 16 * j);
+        w_off[j] = (uint32_t)((r + frow) * ROW_B);
+    }
+}
+
+// Epilogue of one wave.  acc[mi][j][i]: token row = 16*mi + lane%16 of the wave's M range; output column
+// = 16*j + 4*(lane/16) + i of the wave's N range, i.e. a lane holds 4 consecutive columns (8 bytes) of one row per
+// accumulator.  Storing those directly would issue 8-byte writes to 16 different rows per instruction; instead
+// the wave transposes its outputs RPW rows at a time through `ep` (its own RPW * row-bytes of idle LDS) and writes
+// 16 bytes per lane, whole 64/128-byte row segments per 4/8 lanes.  `out` points at the wave's first row and
+// column, rows_here rows of it are valid and cols_here columns (a ragged last N tile).
+template <int MT, int TN, bool SWIGLU, int RPW, bool STREAM>
+__device__ __forceinline__ void store_wave_outputs(const f32x4 (&acc)[2 * MT][TN], uint8_t* ep, int lane, uint16_t* out,
+                                                   int N, int rows_here, int cols_here) {
+    constexpr int CW = SWIGLU ? 8 * TN : 16 * TN;    // output columns of a wave
+    constexpr int RBW = CW * 2;                      // bytes per output row of a wave
+    constexpr int CPR = RBW / 16;                    // 16-byte chunks per row (4 or 8)
+    constexpr int KSH = CPR == 8 ? 0 : 1;            // swizzle key = (row >> KSH) & (CPR-1)
+    constexpr int RPP = 64 / CPR;                    // rows per read-back instruction
+    const int frow = lane & 15, fquad = lane >> 4, rr = lane / CPR, cc = lane % CPR;
+#pragma unroll
+    for (int pass = 0; pass < 32 * MT / RPW; ++pass) {
+#pragma unroll
+        for (int ml = 0; ml < RPW / 16; ++ml) {
+            const int mi = pass * (RPW / 16) + ml;
+            const int r = 16 * ml + frow;
+            uint8_t* erow = ep + r * RBW + (fquad & 1) * 8;
+            const int key = (r >> KSH) & (CPR - 1);
+#pragma unroll
+            for (int jj = 0; jj < (SWIGLU ? TN / 2 : TN); ++jj) {
+                const u32x2 pk = epilogue_pack<SWIGLU>(acc[mi][jj], acc[mi][SWIGLU ? jj + TN / 2 : jj]);
+                *reinterpret_cast<u32x2*>(erow + (((2 * jj + (fquad >> 1)) ^ key) << 4)) = pk;
+            }
+        }
+#pragma unroll
+        for (int ps = 0; ps < RPW / RPP; ++ps) {
+            const int r = rr + RPP * ps;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(ep + r * RBW + ((cc ^ ((r >> KSH) & (CPR - 1))) << 4));
+            if (pass * RPW + r < rows_here && cc * 8 < cols_here) {
+                u32x4* dst = reinterpret_cast<u32x4*>(out + (size_t)(pass * RPW + r) * N + cc * 8);
+                // whole 128-byte lines per 8 lanes can be written non-temporally (the pipeline's next load waits also
+                // cover these stores); half lines per wave stay plain stores, so that L2 merges the halves
+                if (STREAM) __builtin_nontemporal_store(v, dst); else *dst = v;
+            }
+        }
+    }
+}
+
 // MT: 32-row units per wave along M (workgroup rows BM = 64*MT, 2 waves along M)
 // WN: waves along N; 4 -> 8 waves of up to 128x64 outputs, two per SIMD; every wave interleaves
 //     its share of the load / dequantise / LDS-store work with its MFMAs, a piece per MFMA group
@@ -185,37 +285,9 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave & 1, wn = (wave >> 1) % WN;
 
-    // ---- M-tile prefix over experts (exclusive scan of ceil(count/BM)) ----
-    int run = 0;
-    int my_start = 0, my_mt = 0, my_o0 = 0, my_o1 = 0;   // this thread's expert (of the last pass)
-    for (int e0 = 0; e0 < g.E; e0 += NT) {
-        int e = e0 + tid;
-        int mt = 0;
-        if (e < g.E) {
-            my_o0 = g.offsets[e];
-            my_o1 = g.offsets[e + 1];
-            mt = (my_o1 - my_o0 + BM - 1) / BM;
-        }
-        int inc = mt;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            int o = __shfl_up(inc, d);
-            if (lane >= d) inc += o;
-        }
-        if (lane == 63) s_wtot[wave] = inc;
-        __syncthreads();
-        int pre = run, tot = 0;
-#pragma unroll
-        for (int w = 0; w < NT / 64; ++w) {
-            if (w < wave) pre += s_wtot[w];
-            tot += s_wtot[w];
-        }
-        my_start = pre + inc - mt;
-        my_mt = mt;
-        if (e < g.E) s_pref[e] = my_start;
-        run += tot;
-        if (g.E > NT) __syncthreads();   // s_wtot is rewritten by the next pass
-    }
+    // ---- M-tile prefix over experts ----
+    ExpertOfThread mine;
+    const int run = mtile_prefix_scan<NT, BM>(g, tid, s_pref, s_wtot, mine, [](int, int, int) {});
     const int total = run * g.n_tiles_n;
 
     // ---- XCD-aware id: XCD x (= blockIdx % 8) owns tiles [x*per, (x+1)*per) ----
@@ -228,8 +300,8 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     // expert's prefix, tile count and row range: the one that owns q publishes them (one barrier,
     // no search, no second trip to memory for the offsets).  More experts: binary search in LDS.
     if (g.E <= NT) {
-        if (tid < g.E && my_start <= q && q < my_start + my_mt) {
-            s_sel[0] = tid; s_sel[1] = my_start; s_sel[2] = my_mt; s_sel[3] = my_o0; s_sel[4] = my_o1;
+        if (tid < g.E && mine.start <= q && q < mine.start + mine.mt) {
+            s_sel[0] = tid; s_sel[1] = mine.start; s_sel[2] = mine.mt; s_sel[3] = mine.o0; s_sel[4] = mine.o1;
         }
         __syncthreads();
     } else {
@@ -353,13 +425,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     const int fchunk = ((fquad & 1) << 1) | (fquad >> 1);
     constexpr int TM = 2 * MT, TN = 2 * NJ;       // 16-row token tiles / 16-row weight tiles per wave
     uint32_t tok_off[TM], w_off[TN];
-#pragma unroll
-    for (int mi = 0; mi < TM; ++mi) tok_off[mi] = (uint32_t)((wm * 32 * MT + 16 * mi + frow) * ROW_B);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        int r = SWIGLU ? ((j < TN / 2 ? 0 : 128) + wn * (8 * TN) + 16 * (j % (TN / 2))) : (wn * (16 * TN) + 16 * j);
-        w_off[j] = (uint32_t)((r + frow) * ROW_B);
-    }
+    fragment_rows<MT, TN, SWIGLU>(wm, wn, frow, tok_off, w_off);
 
     f32x4 acc[TM][TN];
 #pragma unroll
@@ -495,41 +561,13 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     mfma_sub(NU - 1);
 
     // ---- epilogue ----
-    // acc[mi][j][i]: token row = 16*mi + lane%16 of the wave's M range; output column
-    // = 16*j + 4*(lane/16) + i of the wave's N range, i.e. a lane holds 4 consecutive columns
-    // (8 bytes) of one row per accumulator.  Storing those directly would issue 8-byte writes to
-    // 16 different rows per instruction; instead each wave transposes its outputs through its own
-    // slice of the (now idle) LDS stages and writes 16 bytes per lane, whole 64/128-byte row
-    // segments per 4/8 lanes.  (All waves passed the loop's last barrier, so no one reads the stages.)
+    // All waves passed the loop's last barrier, so no one reads the stages: each wave transposes through its own
+    // slice of them.
     constexpr int CW = SWIGLU ? 8 * TN : 16 * TN;    // output columns of this wave
-    constexpr int RBW = CW * 2;                      // bytes per output row of this wave
-    constexpr int CPR = RBW / 16;                    // 16-byte chunks per row (4 or 8)
-    constexpr int KSH = CPR == 8 ? 0 : 1;            // swizzle key = (row >> KSH) & (CPR-1)
-    uint8_t* ep = ((wave < 4) ? smem0 : smem1) + (wave & 3) * (32 * MT * RBW);
-#pragma unroll
-    for (int mi = 0; mi < TM; ++mi) {
-        const int r = 16 * mi + frow;
-        uint8_t* erow = ep + r * RBW + (fquad & 1) * 8;
-        const int key = (r >> KSH) & (CPR - 1);
-#pragma unroll
-        for (int jj = 0; jj < (SWIGLU ? TN / 2 : TN); ++jj) {
-            const u32x2 pk = epilogue_pack<SWIGLU>(acc[mi][jj], acc[mi][SWIGLU ? jj + TN / 2 : jj]);
-            *reinterpret_cast<u32x2*>(erow + (((2 * jj + (fquad >> 1)) ^ key) << 4)) = pk;
-        }
-    }
-    const int rows_here = min(BM, row_end - row0) - wm * 32 * MT;   // valid rows of this wave
+    uint8_t* ep = ((wave < 4) ? smem0 : smem1) + (wave & 3) * (32 * MT * CW * 2);
     const int ncol0 = n0 + wn * CW;
-    constexpr int RPP = 64 / CPR;                    // rows per pass
-    const int rr = lane / CPR, cc = lane % CPR;
-    if (ncol0 + cc * 8 < N) {
-#pragma unroll
-        for (int ps = 0; ps < 32 * MT / RPP; ++ps) {
-            const int r = rr + RPP * ps;
-            const u32x4 v = *reinterpret_cast<const u32x4*>(ep + r * RBW + ((cc ^ ((r >> KSH) & (CPR - 1))) << 4));
-            if (r < rows_here)
-                *reinterpret_cast<u32x4*>(g.c + (size_t)(row0 + wm * 32 * MT + r) * N + ncol0 + cc * 8) = v;
-        }
-    }
+    store_wave_outputs<MT, TN, SWIGLU, 32 * MT, false>(acc, ep, lane, g.c + (size_t)(row0 + wm * 32 * MT) * N + ncol0, N,
+                                                       min(BM, row_end - row0) - wm * 32 * MT, N - ncol0);
 }
 
 // lane id produced where it is used: the compiler cannot hoist it (and everything derived from it)
@@ -591,41 +629,16 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
     const int wave_s = uni(wave);
     const int wm = wave_s & 1, wn = (wave_s >> 1) % WN;
 
-    int run = 0;
-    int my_start = 0, my_o0 = 0, my_o1 = 0;
-    for (int e0 = 0; e0 < g.E; e0 += NT) {
-        int e = e0 + tid;
-        int mt = 0;
-        if (e < g.E) {
-            my_o0 = g.offsets[e];
-            my_o1 = g.offsets[e + 1];
-            mt = (my_o1 - my_o0 + BM - 1) / BM;
-            s_off[e] = my_o0;
-            if (e == g.E - 1) s_off[g.E] = my_o1;
-            s_ptr[0][e] = (unsigned long long)(uintptr_t)g.b0[e];
-            s_ptr[1][e] = SWIGLU ? (unsigned long long)(uintptr_t)g.b1[e] : 0ull;
-            s_ptr[2][e] = W8 ? (unsigned long long)(uintptr_t)g.s0[e] : 0ull;
-            s_ptr[3][e] = (W8 && SWIGLU) ? (unsigned long long)(uintptr_t)g.s1[e] : 0ull;
-        }
-        int inc = mt;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            int o = __shfl_up(inc, d);
-            if (lane >= d) inc += o;
-        }
-        if (lane == 63) s_wtot[wave] = inc;
-        __syncthreads();
-        int pre = run, tot = 0;
-#pragma unroll
-        for (int w = 0; w < NT / 64; ++w) {
-            if (w < wave) pre += s_wtot[w];
-            tot += s_wtot[w];
-        }
-        my_start = pre + inc - mt;
-        if (e < g.E) s_pref[e] = my_start;
-        run += tot;
-        if (g.E > NT) __syncthreads();
-    }
+    // M-tile prefix over experts; the experts' row offsets and matrix pointers go to LDS tables on the way
+    ExpertOfThread mine;
+    const int run = mtile_prefix_scan<NT, BM>(g, tid, s_pref, s_wtot, mine, [&](int e, int o0, int o1) {
+        s_off[e] = o0;
+        if (e == g.E - 1) s_off[g.E] = o1;
+        s_ptr[0][e] = (unsigned long long)(uintptr_t)g.b0[e];
+        s_ptr[1][e] = SWIGLU ? (unsigned long long)(uintptr_t)g.b1[e] : 0ull;
+        s_ptr[2][e] = W8 ? (unsigned long long)(uintptr_t)g.s0[e] : 0ull;
+        s_ptr[3][e] = (W8 && SWIGLU) ? (unsigned long long)(uintptr_t)g.s1[e] : 0ull;
+    });
     if (tid == 0) s_pref[g.E] = run;
     __syncthreads();
     const int total = run * g.n_tiles_n;
@@ -766,13 +779,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
     const int fchunk = ((fquad & 1) << 1) | (fquad >> 1);
     constexpr int TM = 2 * MT, TN = 2 * NJ;
     uint32_t tok_off[TM], w_off[TN];
-#pragma unroll
-    for (int mi = 0; mi < TM; ++mi) tok_off[mi] = (uint32_t)((wm * 32 * MT + 16 * mi + frow) * ROW_B);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        int r = SWIGLU ? ((j < TN / 2 ? 0 : 128) + wn * (8 * TN) + 16 * (j % (TN / 2))) : (wn * (16 * TN) + 16 * j);
-        w_off[j] = (uint32_t)((r + frow) * ROW_B);
-    }
+    fragment_rows<MT, TN, SWIGLU>(wm, wn, frow, tok_off, w_off);
     f32x4 acc[TM][TN];
     constexpr int TQ = MT / 2;
     constexpr int NP = TM / TQ;
@@ -846,11 +853,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
     __syncthreads();
-    constexpr int CW = SWIGLU ? 8 * TN : 16 * TN;
-    constexpr int RBW = CW * 2;
-    constexpr int CPR = RBW / 16;
-    constexpr int KSH = CPR == 8 ? 0 : 1;
-    constexpr int RPP = 64 / CPR;
+    constexpr int CW = SWIGLU ? 8 * TN : 16 * TN;    // output columns of this wave
     for (;;) {
         const int out_row0 = row0, out_row_end = row_end, out_n0 = n0;
 #pragma unroll
@@ -871,37 +874,13 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
         mfma_sub(NU - 2);
         mfma_sub(NU - 1);
 
-        const int rows_here = min(BM, out_row_end - out_row0) - wm * 32 * MT;
+        // epilogue: stage 0 already holds the next tile; stage 1 is idle until the next tile's first iteration writes
+        // it, so each wave transposes through its 8 KiB slice of stage 1 (64 or 128 rows at a time).  The lane id is
+        // produced here, so that nothing derived from it stays live through the k loop.
         const int ncol0 = out_n0 + wn * CW;
-        const int el = fresh_lane();
-        const int efrow = el & 15, efquad = el >> 4, rr = el / CPR, cc = el % CPR;
-        uint8_t* ep = ((wave_s < 4) ? sA1 : sB1) + (wave_s & 3) * 8192;
-        constexpr int RPW = 8192 / RBW;
-#pragma unroll
-        for (int pass = 0; pass < 32 * MT / RPW; ++pass) {
-#pragma unroll
-            for (int ml = 0; ml < RPW / 16; ++ml) {
-                const int mi = pass * (RPW / 16) + ml;
-                const int r = 16 * ml + efrow;
-                uint8_t* erow = ep + r * RBW + (efquad & 1) * 8;
-                const int key = (r >> KSH) & (CPR - 1);
-#pragma unroll
-                for (int jj = 0; jj < (SWIGLU ? TN / 2 : TN); ++jj) {
-                    const u32x2 pk = epilogue_pack<SWIGLU>(acc[mi][jj], acc[mi][SWIGLU ? jj + TN / 2 : jj]);
-                    *reinterpret_cast<u32x2*>(erow + (((2 * jj + (efquad >> 1)) ^ key) << 4)) = pk;
-                }
-            }
-#pragma unroll
-            for (int ps = 0; ps < RPW / RPP; ++ps) {
-                const int r = rr + RPP * ps;
-                const u32x4 v = *reinterpret_cast<const u32x4*>(ep + r * RBW + ((cc ^ ((r >> KSH) & (CPR - 1))) << 4));
-                if (pass * RPW + r < rows_here && ncol0 + cc * 8 < N)
-                {
-                    u32x4* dst = reinterpret_cast<u32x4*>(g.c + (size_t)(out_row0 + wm * 32 * MT + pass * RPW + r) * N + ncol0 + cc * 8);
-                    if (SWIGLU) *dst = v; else __builtin_nontemporal_store(v, dst);
-                }
-            }
-        }
+        store_wave_outputs<MT, TN, SWIGLU, 8192 / (CW * 2), !SWIGLU>(
+            acc, ((wave_s < 4) ? sA1 : sB1) + (wave_s & 3) * 8192, fresh_lane(),
+            g.c + (size_t)(out_row0 + wm * 32 * MT) * N + ncol0, N, min(BM, out_row_end - out_row0) - wm * 32 * MT, N - ncol0);
         if (!more) return;
         __syncthreads();
     }
