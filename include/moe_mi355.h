@@ -136,9 +136,11 @@ int moe_dispatch_static(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k
  * on bf16 MFMA with fp32 accumulation.
  *   x         device bf16: rows of the sorted token matrix [n_rows, h]; or, when
  *             row_map != NULL, the unsorted matrix, row r being x[row_map[r]]
- *   x_rows    rows of x (>= 1).  It bounds the gather: a row_map entry outside [0, x_rows) reads a row
- *             of zeros where the descriptor-based loads are used (x smaller than 4 GiB) and is
- *             undefined otherwise; without row_map it only has to cover the rows the call reads
+ *   x_rows    rows of x (>= 1).  It bounds the gather where rows are fetched through a buffer
+ *             descriptor (256-row tiles, x smaller than 4 GiB): a row_map entry outside [0, x_rows)
+ *             then reads zeros (or, once its byte offset wraps 32 bits, some row of x), never memory
+ *             outside x; on the other paths such an entry is undefined.  Without row_map it only has
+ *             to cover the rows the call reads
  *   row_map   device int32 [n_rows] or NULL
  *   w_gate/w_up/w_down   device arrays of E device pointers: Wg_e, Wu_e bf16
  *             [I, h]; Wd_e bf16 [h, I]  (nn.Linear [out, in] layout)
