@@ -236,6 +236,39 @@ def test_expert_sub_range_through_the_persistent_kernel(fp8):
     assert (y[:a] == 7.0).all() and (y[b:] == 7.0).all()
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("E,h,I,counts", [
+    (2, 128, 128, [300, 260]),                # two k-stages: the shortest pipeline the persistent kernel runs
+    (2, 128, 384, [513, 256]),                # gate/up: 2 stages; down: 6; a tile of one row
+    (3, 256, 128, [700, 0, 300]),             # down projection with 2 stages, an empty expert in between
+    (512, 128, 128, [200] * 512),             # as many experts as the kernel keeps tables for
+])
+def test_persistent_kernel_corner_shapes(fp8, E, h, I, counts):
+    """The 256-row persistent kernel (mean rows per expert >= 192, K a multiple of 128) at the ends of what
+    it accepts; rows gathered through a row map."""
+    print(f"persistent corners fp8={fp8} E={E} h={h} I={I}", flush=True)
+    y, ref32, _ = run_case(E, h, I, counts, fp8, seed=37, use_row_map=True)
+    assert np.isfinite(y).all() and rel_max(y, ref32) <= TOL
+
+
+def test_row_map_may_repeat_rows():
+    """Several sorted rows may name the same source row (a token routed to k experts)."""
+    from moe_gen_amd import ops
+    h, I, n_src, n = 256, 256, 100, 600
+    ws, ptrs = _one_expert(h, I, 51)
+    g = torch.Generator().manual_seed(52)
+    x = torch.randn(n_src, h, generator=g).to(torch.bfloat16)
+    rm = torch.randint(0, n_src, (n,), generator=g, dtype=torch.int32)
+    off = torch.tensor([0, n], dtype=torch.int32, device="cuda")
+    y = ops.grouped_swiglu(x.cuda(), rm.cuda(), ptrs, off, n)
+    y_src = ops.grouped_swiglu(x.cuda(), None, ptrs, torch.tensor([0, n_src], dtype=torch.int32, device="cuda"), n_src)
+    torch.cuda.synchronize()
+    wg, wu, wd = (O.bf16_to_f32(bits(w)) for w in ws)
+    ref32 = O.mlp_f32(O.bf16_to_f32(bits(x)), wg, wu, wd)[rm.long().numpy()]
+    assert rel_max(O.bf16_to_f32(bits(y)), ref32) <= TOL
+    assert np.array_equal(bits(y), bits(y_src)[rm.long().numpy()])       # a row's result does not depend on its tile
+
+
 def test_grouped_single_expert_is_plain_mlp():
     """E = 1 reduces to a dense SwiGLU MLP: compare with torch's own bf16 linear layers on the GPU."""
     from moe_gen_amd import DeepseekV3Config, DeepseekV3MLP
