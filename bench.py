@@ -81,10 +81,10 @@ def cpu_baseline(w, blk, n_sample: int, passes: int = 3):
                       "stock-PyTorch CPU restatement of the reference block"}
 
 
-def staged_run(w, blk, x, steps: int, routing_aware: bool = False):
+def staged_run(w, blk, x, steps: int, routing_aware: bool = False, pool: int = 0):
     """Second figure: the same block with every expert matrix in pinned host memory, delivered by
-    the stager (cyclic prefetch on the copy stream, event hand-off) while the previous layer
-    computes.  Two layers' worth of modules alternate so that copies overlap compute, as in a model.
+    the stager (cyclic prefetch on the copy stream, event hand-off) into a pool of `pool` slots while
+    earlier experts are multiplied.  Two layers' worth of modules alternate, as in a model.
     routing_aware: copy only the experts that received tokens, busiest first, once the per-expert
     counts are known (fewer bytes, but the copies cannot start before the router has run)."""
     import time as _t
@@ -96,7 +96,9 @@ def staged_run(w, blk, x, steps: int, routing_aware: bool = False):
     wdt = torch.float8_e4m3fn if w.fp8 else torch.bfloat16
     names = blk.experts[0].names
     shapes = {"routed_expert": {f"{n}.weight": (tuple(getattr(blk.experts[0], n).weight.shape), wdt) for n in names}}
-    n_slots = {"routed_expert": 2 * E}
+    # the reference engine's prefill pool holds 20 routed experts (deepseekv3_initializer.py:912-916); a layer
+    # with more experts runs in waves of half the pool while the other half is being filled
+    n_slots = {"routed_expert": pool if pool > 0 else min(20, 2 * E)}
     has_shared = bool(w.S) and w.family != "mixtral"
     if has_shared:
         shapes["shared_expert"] = {f"{n}.weight": (tuple(getattr(blk.shared_experts, n).weight.shape), wdt) for n in names}
@@ -309,8 +311,9 @@ def run_workload(name: str, args, with_cpu: bool):
     if args.decoder_half:
         result["decoder_half"] = decoder_half_run(w, blk, x, args.steps)
     if args.staged:
-        result["staged"] = staged_run(w, blk, x, max(2, args.steps // 2))
-        result["staged_routing_aware"] = staged_run(w, blk, x, max(2, args.steps // 2), routing_aware=True)
+        result["staged"] = staged_run(w, blk, x, max(2, args.steps // 2), pool=args.staged_pool)
+        result["staged_routing_aware"] = staged_run(w, blk, x, max(2, args.steps // 2), routing_aware=True, pool=args.staged_pool)
+        result["staged"]["pool_slots"] = result["staged_routing_aware"]["pool_slots"] = args.staged_pool or min(20, 2 * w.E)
     if with_cpu:
         # full size where the workload is small (DeepSeek-V2-Lite 4096 tokens, the 256-token decode case),
         # a bounded sample of the first tokens elsewhere
@@ -421,6 +424,7 @@ def main():
                     "reading them through the row map inside the GEMM")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--staged", action="store_true", help="also time the block with weights staged from pinned host memory")
+    ap.add_argument("--staged-pool", type=int, default=0, help="routed-expert slots of the staging pool (default 20, the reference engine's prefill default)")
     ap.add_argument("--decoder-half", action="store_true", help="also time RMSNorm + block + residual add, fused and separate")
     ap.add_argument("--cpu-sample", type=int, default=1024, help="tokens of the workload the CPU baseline runs")
     ap.add_argument("--ceiling", action="store_true", help="instead of the benchmark: registers-only MFMA rate, vendor dense "

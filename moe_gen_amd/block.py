@@ -192,20 +192,23 @@ def pool_size(expert, module_type: str = "routed_expert") -> int:
 
 
 def expert_waves(n_experts: int, pool: int, hot=None):
-    """Cut a layer's experts into waves that fit a pool of `pool` slots.
+    """Cut a layer's experts into waves for a pool of `pool` slots.
 
     Returns a list of (first, last_plus_one, fetch_list): the grouped kernels of a wave run on the
     experts [first, last_plus_one) and `fetch_list` names the ones whose weights the wave holds.
-    Without `hot` every expert is fetched, in id order, `pool` at a time -- the order in which the
-    reference's copy worker delivers them (HtoD_Engine.cpp:201-268), so a wave's weights are
-    exactly what the pool holds or receives next.  With `hot` (ids of the experts that received
-    tokens, on-demand staging) only those are fetched; a wave then spans from its first to its
-    last hot expert and the cold ones in between own no rows."""
+    Experts that fit the pool at once are one wave.  Otherwise a wave takes HALF the pool, so that the
+    engine copies the next wave into the other half while this one is multiplied -- the overlap the
+    reference gets from fetching, using and freeing one expert at a time against a pool that its copy
+    worker keeps filling (Wrapper.py:475-521, HtoD_Engine.cpp:201-268); with waves as large as the pool
+    every copy would wait for a release and every launch for a copy.
+    Without `hot` every expert is fetched, in id order -- the order in which the copy worker delivers
+    them, so a wave's weights are exactly what the pool holds or receives next.  With `hot` (ids of the
+    experts that received tokens, on-demand staging) only those are fetched; a wave then spans from its
+    first to its last hot expert and the cold ones in between own no rows."""
     pool = max(1, int(pool))
-    if hot is None:
-        return [(a, min(a + pool, n_experts), list(range(a, min(a + pool, n_experts)))) for a in range(0, n_experts, pool)]
-    hot = sorted(hot)
-    return [(hot[i], hot[min(i + pool, len(hot)) - 1] + 1, hot[i:i + pool]) for i in range(0, len(hot), pool)]
+    ids = list(range(n_experts)) if hot is None else sorted(hot)
+    step = pool if len(ids) <= pool else max(1, pool // 2)
+    return [(ids[i], ids[min(i + step, len(ids)) - 1] + 1, ids[i:i + step]) for i in range(0, len(ids), step)]
 
 
 def staged_experts_forward(experts, launch, counts_host=None, on_demand=False, stream_wait=None, module_type="routed_expert"):
@@ -244,9 +247,12 @@ def staged_experts_forward(experts, launch, counts_host=None, on_demand=False, s
     if len(waves) > 1 and counts_host is None:
         raise RuntimeError("staged_experts_forward: more than one wave needs the per-expert counts on the host")
     ordered = bool(getattr(eng, "stream_ordered_release", False))
-    for a, b, fetch in waves:
-        if hot is not None and len(hot) > pool:
-            eng.fetch([experts[e].expert_weights_idx for e in fetch])
+    on_demand_waves = hot is not None and len(hot) > pool
+    if on_demand_waves:                                      # the first wave's copies; each wave then asks for the next one's
+        eng.fetch([experts[e].expert_weights_idx for e in waves[0][2]])
+    for w, (a, b, fetch) in enumerate(waves):
+        if on_demand_waves and w + 1 < len(waves):           # into the half of the pool this wave does not hold
+            eng.fetch([experts[e].expert_weights_idx for e in waves[w + 1][2]])
         got = {e: _tensors_of(experts[e], eng.get_weights(experts[e].expert_weights_idx)) for e in fetch}
         stand_in = got[fetch[0]]                             # an expert without rows is never read
         rows = [got.get(e, stand_in) for e in range(a, b)]

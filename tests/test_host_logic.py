@@ -168,8 +168,9 @@ def test_engine_pool_smaller_than_the_layer_runs_in_waves(E, slots):
         eng.synced = True
 
     block.staged_experts_forward(experts, launch, counts, stream_wait=stream_wait)
-    assert [a for a, _, _ in launches] == list(range(0, E, slots))
-    assert launches[-1][1] == E and all(b - a <= slots for a, b, _ in launches)
+    step = slots if E <= slots else max(1, slots // 2)       # half the pool per wave: the other half is being copied
+    assert [a for a, _, _ in launches] == list(range(0, E, step))
+    assert launches[-1][1] == E and all(b - a <= step for a, b, _ in launches)
     assert [n for _, _, n in launches] == [sum(counts[a:b]) for a, b, _ in launches]
     assert not eng.held and eng.calls[0] == ("clear", L, 0)
     gets = [c[1] for c in eng.calls if c[0] == "get"]
@@ -189,8 +190,10 @@ def test_engine_phase_and_unknown_pool():
     assert block.pool_size(DecodingWrapped(eng, 0, 0, _engine_config(2, 4))) == 4
     assert block.pool_size(_Wrapped(eng, 0, 0, _engine_config(2, 4))) == 2
     assert block.pool_size(_Wrapped(eng, 0, 0)) == 1          # nothing known: one at a time, as Wrapper.py:475-521
-    assert block.expert_waves(5, 2) == [(0, 2, [0, 1]), (2, 4, [2, 3]), (4, 5, [4])]
-    assert block.expert_waves(9, 2, hot=[7, 1, 4]) == [(1, 5, [1, 4]), (7, 8, [7])]
+    assert block.expert_waves(2, 2) == [(0, 2, [0, 1])]                                   # fits the pool: one wave
+    assert block.expert_waves(5, 4) == [(0, 2, [0, 1]), (2, 4, [2, 3]), (4, 5, [4])]     # else half the pool per wave
+    assert block.expert_waves(3, 1) == [(0, 1, [0]), (1, 2, [1]), (2, 3, [2])]
+    assert block.expert_waves(9, 4, hot=[7, 1, 4, 8, 2]) == [(1, 3, [1, 2]), (4, 8, [4, 7]), (8, 9, [8])]
 
 
 def test_on_demand_waves_fetch_only_experts_with_tokens():
@@ -203,7 +206,7 @@ def test_on_demand_waves_fetch_only_experts_with_tokens():
     counts = [0, 3, 0, 0, 9, 1, 0, 2, 0, 0, 5, 0]
     launches = []
     block.staged_experts_forward(experts, lambda rows, a, b, n: launches.append((a, b, n)), counts, on_demand=True)
-    assert launches == [(1, 6, 13), (7, 11, 7)]
+    assert launches == [(1, 2, 3), (4, 5, 9), (5, 6, 1), (7, 8, 2), (10, 11, 5)]     # 5 hot experts, 3 slots: one per wave
     assert [c[1] for c in eng.calls if c[0] == "get"] == [f"routed_expert_{L}_{e}" for e in (1, 4, 5, 7, 10)]
     eng.calls.clear()
     few = [0, 0, 4, 0, 0, 0, 0, 0, 6, 0, 0, 0]                # fits the pool: one wave, busiest first
