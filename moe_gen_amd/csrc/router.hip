@@ -529,6 +529,131 @@ __global__ __launch_bounds__(64 * WE * WT) void router_kernel(
     }
 }
 
+// Third logit engine, for up to 16 experts and few tokens: one lane per (token, expert) pair on the vector
+// ALU.  A chain of dependent 4x4 MFMAs advances one k in 14 cycles (measured: registers only) whatever the
+// instruction's 256 outputs are used for, 26 with its operand reads, so a launch of a few thousand tokens
+// takes h * 26 cycles on a handful of CUs (Mixtral-8x22B, 256 tokens: 72 us).  v_fmac_f32 is the same
+// single fused multiply-add per k, the canonical order, at 9 cycles per dependent step (18 with the
+// operand reads: a 16-byte LDS read costs the wave about 16 cycles of issue, whatever the read-ahead), and
+// 64 pairs per wave spread a small launch over 4 to 8 times as many CUs: 51 us for the same launch.  A
+// workgroup is ONE wave: 64 / EBW tokens x EBW (8 or 16, padded) experts; operands go through two LDS
+// stages as fp32 (a lane reads 16 bytes of its token's row and of its expert's row per 4 k); with a single
+// wave the LDS executes its accesses in program order, so the k loop needs no barrier.  The staging of
+// stage st+1 (two stages ahead in registers) is spread between the multiply-adds of stage st.
+template <int EBW>
+__global__ __launch_bounds__(64) void router_pair_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ wg, const float* __restrict__ bias,
+    moe_router_params p, int32_t* __restrict__ topk_idx, float* __restrict__ topk_w, float* __restrict__ logits_out) {
+    constexpr int TBW = 64 / EBW;            // tokens per workgroup
+    constexpr int KC = 128, LDK = KC + 4;    // k per stage; padded fp32 row stride: conflict-free 16-byte reads
+    constexpr int ROWS = TBW + EBW;
+    constexpr int CH = ROWS * (KC / 8);      // 16-byte bf16 chunks per stage
+    constexpr int CPT = (CH + 63) / 64;
+    __shared__ __attribute__((aligned(16))) float st0[ROWS * LDK];
+    __shared__ __attribute__((aligned(16))) float st1[ROWS * LDK];
+    const int lane = threadIdx.x, tl = lane / EBW, el = lane % EBW;
+    const int n = p.n_tokens, h = p.hidden, E = p.n_experts;
+    const int t0 = blockIdx.x * TBW;
+
+    // chunk lane + 64 i of a stage: row (lane + 64 i) / 16 (tokens first, then experts), 8 k from (chunk % 16) * 8
+    const uint16_t* src[CPT];
+    int kc[CPT], dst[CPT];
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+        const int c = lane + 64 * i, row = min(c / (KC / 8), ROWS - 1);
+        kc[i] = (c % (KC / 8)) * 8;
+        src[i] = row < TBW ? x + (size_t)min(t0 + row, n - 1) * h : wg + (size_t)min(row - TBW, E - 1) * h;
+        dst[i] = row * LDK + kc[i];
+    }
+    u32x4 r[2][CPT];
+    // loads are unconditional (clamped addresses, chunks past h are zeroed on their way to LDS): a load under a
+    // branch makes the compiler wait for every outstanding load at the next use
+    auto load = [&](int set, int i, int k0) {
+        const int k = k0 + kc[i];
+        r[set][i] = *reinterpret_cast<const u32x4*>(src[i] + (k < h ? k : 0));
+    };
+    auto piece = [&](int i, int set, float* buf, int k0, int k0_next) {
+        const u32x4 v = k0 + kc[i] < h ? r[set][i] : u32x4{0, 0, 0, 0};
+        if (lane + 64 * i < CH) {
+            f32x4 lo, hi;
+            lo[0] = __uint_as_float(v[0] << 16); lo[1] = __uint_as_float(v[0] & 0xffff0000u);
+            lo[2] = __uint_as_float(v[1] << 16); lo[3] = __uint_as_float(v[1] & 0xffff0000u);
+            hi[0] = __uint_as_float(v[2] << 16); hi[1] = __uint_as_float(v[2] & 0xffff0000u);
+            hi[2] = __uint_as_float(v[3] << 16); hi[3] = __uint_as_float(v[3] & 0xffff0000u);
+            *reinterpret_cast<f32x4*>(buf + dst[i]) = lo;
+            *reinterpret_cast<f32x4*>(buf + dst[i] + 4) = hi;
+        }
+        load(set, i, k0_next);
+    };
+
+    float acc = 0.0f;
+    const int a_off = tl * LDK, b_off = (TBW + el) * LDK;
+        constexpr int NK4 = KC / 4, AHEAD = 6;    // operand reads run AHEAD steps of 4 k in front of their multiply-adds
+    auto multiply_and_stage = [&](const float* rd, float* wr, int set, int k0, int k0_next) {
+        f32x4 a[NK4], b[NK4];
+#pragma unroll
+        for (int k4 = 0; k4 < AHEAD; ++k4) {
+            a[k4] = *reinterpret_cast<const f32x4*>(rd + a_off + k4 * 4);
+            b[k4] = *reinterpret_cast<const f32x4*>(rd + b_off + k4 * 4);
+        }
+#pragma unroll
+        for (int k4 = 0; k4 < NK4; ++k4) {
+            if (k4 + AHEAD < NK4) {
+                a[k4 + AHEAD] = *reinterpret_cast<const f32x4*>(rd + a_off + (k4 + AHEAD) * 4);
+                b[k4 + AHEAD] = *reinterpret_cast<const f32x4*>(rd + b_off + (k4 + AHEAD) * 4);
+            }
+#pragma unroll
+            for (int i = k4 * CPT / NK4; i < (k4 + 1) * CPT / NK4; ++i) piece(i, set, wr, k0, k0_next);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk)   // as volatile asm the chain stays between its operand reads (plain arithmetic
+                                             // sinks to the end of the stage, and every operand of the stage is spilled)
+                asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(acc) : "v"(a[k4][kk]), "v"(b[k4][kk]));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    const int nstage = (h + KC - 1) / KC;
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) load(0, i, 0);
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) load(1, i, min(1, nstage - 1) * KC);
+    // register set s holds stage st + 1 while stage st (parity s ^ 1) is multiplied, the other set stage st + 2
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) piece(i, 0, st0, 0, min(2, nstage - 1) * KC);
+    int st = 0;
+    for (; st + 1 < nstage; st += 2) {
+        multiply_and_stage(st0, st1, 1, (st + 1) * KC, min(st + 3, nstage - 1) * KC);
+        multiply_and_stage(st1, st0, 0, (st + 2) * KC, min(st + 4, nstage - 1) * KC);
+    }
+    if (st < nstage) multiply_and_stage(st0, st1, 1, (st + 1) * KC, (nstage - 1) * KC);
+
+    __syncthreads();                          // (one wave: orders the operand reads before the logits overwrite them)
+    float* lg = st0;
+    lg[tl * EBW + el] = acc;
+    __syncthreads();
+    // selection: 16 lanes per token, as in router_kernel for up to 16 experts
+#pragma unroll
+    for (int tb = 0; tb < TBW; tb += 4) {
+        if (t0 + tb >= n) break;
+        const int tg = tb + lane / 16, t = t0 + tg;
+        const bool live = tg < TBW && t < n;
+        const int tr = live ? t : min(t0 + tb, n - 1), tlr = live ? tg : tb;
+        route_token<16, 1>(lg + tlr * EBW, bias, p, topk_idx + (size_t)tr * p.top_k, topk_w + (size_t)tr * p.top_k,
+                           logits_out ? logits_out + (size_t)tr * E : nullptr, live);
+    }
+}
+
+template <int EBW>
+int launch_pairs(const void* x, const void* w, const float* bias, const moe_router_params& p, int32_t* idx, float* tw,
+                 float* lo, hipStream_t st) {
+    constexpr int TBW = 64 / EBW;
+    hipLaunchKernelGGL((router_pair_kernel<EBW>), dim3((p.n_tokens + TBW - 1) / TBW), dim3(64), 0, st, (const uint16_t*)x,
+                       (const uint16_t*)w, bias, p, idx, tw, lo);
+    MOE_HIP_CHECK(hipGetLastError());
+    return MOE_OK;
+}
+
 template <bool SMALL, int TG, int NEB, int WE, int WT, int GW, int NX = 0>
 int launch(const void* x, const void* w, const float* bias, const moe_router_params& p, int32_t* idx,
            float* tw, float* lo, const NormArgs& nrm, hipStream_t st) {
@@ -621,6 +746,11 @@ int route(const void* x, const void* w_gate, const float* bias, const moe_router
     //                 12288: 0.374, 0.479
     //   256 experts   1024 tokens: 4x64 0.165, 16x16 0.231, 64x4 0.583;  8192: 16x16 0.519, 32x32 0.657;
     //                 12288: 0.775, 0.683
+    // up to 16 experts and few tokens: a lane per (token, expert) pair
+    // measured (us, h = 4096; pairs / 4x4 engine): 8 experts 256 tokens 35 / 50, 8192: 42 / 53, 16384: 58 / 61,
+    // 32768: 122 / 89; 16 experts 4096 tokens: 41 / 50, 8192: 81 / 53
+    if (E <= 8 && n <= 8192 && !nrm.w) return launch_pairs<8>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    if (E <= 16 && n <= 4096 && !nrm.w) return launch_pairs<16>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
     if (E <= 64) {
         if (n <= (E <= 32 ? 32768 : 24576)) {   // 16 tokens per workgroup, 16 experts per wave
             if (E <= 16) MOE_ROUTE(true, 4, 1, 1, 1, 16);

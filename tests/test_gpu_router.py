@@ -127,8 +127,8 @@ def test_every_expert_count_bracket(E):
     """One case per kernel instantiation (and an odd count inside it): greedy softmax routing and,
     where the count allows groups, sigmoid group-limited routing; logits, indices and weights
     bit-for-bit.  The token count picks the logit engine and its block layout inside a bracket:
-    150 tokens (full tiles and a ragged one) the 4x4 MFMA engine with 16 tokens per workgroup, or
-    with 4 above 128 experts; 4100 tokens (more than 128 experts) 16 per workgroup; 8200 tokens
+    150 tokens (full tiles and a ragged one) the vector-ALU engine with a lane per (token, expert) pair up to
+    16 experts, above that the 4x4 MFMA engine with 16 tokens per workgroup, or with 4 above 128 experts; 4100 tokens (more than 128 experts) 16 per workgroup; 8200 tokens
     (more than 64 experts) the 32x32 MFMA engine (129 to 208 experts: with extra 4-expert groups per wave); up to 64 experts 33000 tokens the 4x4 engine with
     64 tokens per workgroup and 65600 the 32x32 engine (always 4x4 up to 16 experts)."""
     print(f"router bracket E={E}", flush=True)
@@ -163,10 +163,10 @@ def test_router_random_shapes_at_switch_points():
     every switch point of the logit engine's dispatch, bit-for-bit against the oracle."""
     import random
     rng = random.Random(7)
-    edges = [1, 3, 4, 5, 15, 16, 17, 63, 64, 65, 1023, 1024, 1025, 8191, 8192, 8193, 24576, 24577, 32768,
+    edges = [1, 3, 4, 5, 7, 8, 9, 15, 16, 17, 63, 64, 65, 1023, 1024, 1025, 4095, 4096, 4097, 8191, 8192, 8193, 24576, 24577, 32768,
              32769, 65536, 65537]
-    for it in range(40):
-        E = rng.choice([1, 3, 7, 9, 16, 20, 31, 32, 40, 50, 64, 72, 96, 120, 129, 160, 190, 208, 240, 256])
+    for it in range(56):
+        E = rng.choice([1, 3, 7, 8, 9, 16, 20, 31, 32, 40, 50, 64, 72, 96, 120, 129, 160, 190, 208, 240, 256])
         k = rng.randint(1, min(E, 8))
         fam = rng.choice(["v2_greedy", "v2_group", "v3", "mixtral"])
         divs = [g for g in (2, 4, 8, 16) if E % g == 0 and E // g >= 2]
