@@ -333,7 +333,9 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     // and crowd a few memory channels.  N tile t walks k from stage t instead (mod nk; a dot product does not care
     // where it starts, and a column's order depends on nothing but its position): Mixtral-8x22B, 256 tokens, down
     // projection 0.302 -> 0.273 ms, gate/up 0.640 -> 0.620 ms.
-    const int rot = MT < 4 ? n_tile % nk : 0;
+    // fp8 weights under these tiles are fetched 128 k at a time (see PAIR8 below): pairs of stages stay together
+    constexpr bool PAIR8 = W8 && MT < 4;
+    const int rot = MT < 4 ? (PAIR8 ? (2 * n_tile) % nk : n_tile % nk) : 0;
     auto stage_at = [&](int kt) { const int kp = kt + rot; return kp >= nk ? kp - nk : kp; };
 
     // ---- per-thread load coordinates ----
@@ -388,11 +390,61 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     constexpr int PF = (MT <= 2) ? 2 : 1;
     u32x4 ra[PF][NA], rb[PF][NB];
     float rs[PF][2];
+
+    // PAIR8.  A 64-k stage of fp8 weights is 64 bytes of a row, half a cache line: fetched stage by stage, every
+    // row costs two half-line requests, and a CU can only keep so many requests in flight whatever their size
+    // (DeepSeek-V3 shapes, 8 rows per expert: 3.6 TB/s of weights against 5-6.5 with bf16 weights).  So the
+    // weights of TWO stages are requested together, 8 lanes x 16 bytes = one whole line per row: thread (row
+    // tid/8 + 64 i, i < 4; 16-byte chunk c = tid%8) gets 16 weights of stage c/4 of the pair.  Lanes c and c^4
+    // then swap their second 8 bytes, after which every lane holds 8 weights of either stage (one 16-byte LDS
+    // store each, the unit of work of a data item): chunk 2 (c%4) + (c/4 ^ stage) of the stage's LDS row.  Two
+    // register sets of pairs; a set is refilled while the second stage of its pair is stored, three
+    // iterations before it is needed again.
+    const int prow = tid >> 3, pq = tid & 3, phb = (tid >> 2) & 1;
+    u32x4 rp[2][4];
+    float rps[2][2];
+    int p_n[4];
+    uint32_t p_lds[2];
+    if (PAIR8) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = prow + 64 * i;
+            p_n[i] = min(SWIGLU ? n0 + (r & 127) : n0 + r, N - 1);
+        }
+#pragma unroll
+        for (int st = 0; st < 2; ++st) p_lds[st] = (uint32_t)(prow * ROW_B + (((2 * pq + (phb ^ st)) ^ swz(prow)) << 4));
+    }
+    const int npair = nk >> 1, prot = rot >> 1;
+    auto pair_load = [&](int pr_pipe, int ps, int i) {      // chunk i of pair pr_pipe (pipeline order) into set ps
+        const bool past = pr_pipe >= npair;                  // nobody reads it: not from the weights
+        int pr = min(pr_pipe, npair - 1) + prot;
+        pr = pr >= npair ? pr - npair : pr;
+        const uint8_t* m = (SWIGLU && i >= 2) ? bmat1 : bmat0;
+        rp[ps][i] = gload16_w<true>(past ? (const uint8_t*)g.a : m + (size_t)p_n[i] * K + (size_t)pr * 128 + ((tid & 7) << 4));
+        if (i == 1) rps[ps][0] = sc0[srow0 + pr];
+        if (i == 3) rps[ps][1] = sc1[srow1 + pr];
+    };
+    auto pair_swap = [&](int ps, int i) {                    // lanes c and c^4 swap dwords 2, 3
+        const u32x4 own = rp[ps][i];
+        u32x4 o;
+        // first stage of the pair: c < 4 keeps its dwords 0, 1; c >= 4 takes dwords 2, 3 of lane c-4 (row_shr:4, banks 1, 3)
+        o[0] = (uint32_t)__builtin_amdgcn_update_dpp((int)own[0], (int)own[2], 0x114, 0xf, 0xa, false);
+        o[1] = (uint32_t)__builtin_amdgcn_update_dpp((int)own[1], (int)own[3], 0x114, 0xf, 0xa, false);
+        // second stage: c >= 4 keeps its dwords 0, 1; c < 4 takes dwords 2, 3 of lane c+4 (row_shl:4, banks 0, 2)
+        o[2] = (uint32_t)__builtin_amdgcn_update_dpp((int)own[0], (int)own[2], 0x104, 0xf, 0x5, false);
+        o[3] = (uint32_t)__builtin_amdgcn_update_dpp((int)own[1], (int)own[3], 0x104, 0xf, 0x5, false);
+        rp[ps][i] = o;
+    };
+    auto pair_store = [&](uint8_t* Bs, int ps, int i, int st) {   // the 8 weights of stage st of the pair -> LDS
+        const u32x4 o = dequant8(rp[ps][i][2 * st], rp[ps][i][2 * st + 1], rps[ps][i >> 1]);
+        *reinterpret_cast<u32x4*>(Bs + p_lds[st] + i * 64 * ROW_B) = o;
+    };
     auto gload = [&](int kt_pipe, int set) {
         const int kt = stage_at(kt_pipe);
         const size_t kofs = (size_t)kt * BK;
 #pragma unroll
         for (int i = 0; i < NA; ++i) ra[set][i] = gload16(g.a + (size_t)a_src[i] * K + kofs + lchunk * 8);
+        if (PAIR8) return;
 #pragma unroll
         for (int i = 0; i < NB; ++i) {
             const uint8_t* m = (SWIGLU && i >= NB / 2) ? bmat1 : bmat0;  // rows >= 128 of the B tile are the up matrix
@@ -407,7 +459,13 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
         uint8_t* Bs = As + A_STAGE;
 #pragma unroll
         for (int i = 0; i < NA; ++i) *reinterpret_cast<u32x4*>(As + a_lds + i * RA * ROW_B) = ra[set][i];
-        if (W8) {
+        if (PAIR8) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                pair_swap(0, i);
+                pair_store(Bs, 0, i, 0);
+            }
+        } else if (W8) {
 #pragma unroll
             for (int i = 0; i < NB; ++i) {
                 u32x4 l, h;
@@ -479,6 +537,12 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     // kt+PF (possibly still in flight).  The iteration moves tile kt+1 into the other LDS stage,
     // refills that register set with tile kt+1+PF and multiplies tile kt.
     gload(0, 0);
+    if (PAIR8) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pair_load(0, 0, i);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pair_load(1, 1, i);
+    }
     lds_store(smem0, 0);
     // No load or store of the pipeline sits under a branch or in a region that only some waves
     // execute (past the end the last tile is loaded again and stored where nobody reads it): with
@@ -494,9 +558,10 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     // tile kt+1+PF.  The items are spread over the iteration, one per group of MFMAs, so LDS, the
     // vector-memory pipe and the matrix core see a steady mix instead of bursts; with exact load
     // waits each item stalls only until its own chunk (requested PF iterations earlier) is there.
-    constexpr int NBI = W8 ? 2 * NB : NB;
+    constexpr int NBI = W8 ? 2 * NB : NB;      // (PAIR8: 4 rows, which is the same number)
     constexpr int NI = NA + NBI;
-    auto data_item = [&](int i, uint8_t* As, int kt, int set) {
+    // par = kt & 1 and ps, the register set of the pair that stage kt+1 belongs to, are literals at the call sites
+    auto data_item = [&](int i, uint8_t* As, int kt, int set, int par, int ps) {
         uint8_t* Bs = As + A_STAGE;
         const int kn = stage_at(min(kt + 1 + PF, nk - 1));
         const size_t kofs = (size_t)kn * BK;
@@ -506,6 +571,15 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
         if (i < NA) {
             *reinterpret_cast<u32x4*>(As + a_lds + i * RA * ROW_B) = ra[set][i];
             ra[set][i] = gload16(g.a + (size_t)a_src[i] * K + kofs + lchunk * 8);
+        } else if (PAIR8) {
+            const int b = i - NA;
+            if (par) {                      // stage kt+1 opens a pair
+                pair_swap(ps, b);
+                pair_store(Bs, ps, b, 0);
+            } else {                        // it closes one: the set is free for the pair after the next
+                pair_store(Bs, ps, b, 1);
+                pair_load((kt >> 1) + 2, ps, b);
+            }
         } else if (W8) {
             const int b = (i - NA) >> 1, half = (i - NA) & 1;
             const uint8_t* m = (SWIGLU && b >= NB / 2) ? bmat1 : bmat0;
@@ -527,7 +601,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     };
     constexpr int NG = NU;                        // one group of MFMAs per slot
     constexpr int WPS = TN / NP;                  // weight fragments of the second k-step read per slot
-    auto iteration = [&](int kt, int set, int par) {   // par == kt & 1
+    auto iteration = [&](int kt, int set, int par, int ps = 0) {   // par == kt & 1
         const uint8_t* rd = par ? smem1 : smem0;
         uint8_t* wr = par ? smem0 : smem1;
 #pragma unroll
@@ -537,7 +611,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
 #pragma unroll
             for (int i0 = v * NI / NG; i0 < (v + 1) * NI / NG; ++i0) {
                 const int i = (W8 && NA == 4 && NI == 8) ? ((i0 & 1) ? NA + (i0 >> 1) : (i0 >> 1)) : i0;
-                data_item(i, wr, kt, set);
+                data_item(i, wr, kt, set, par, ps);
             }
             if (!W8) __builtin_amdgcn_sched_barrier(0);
             if (v >= 2) mfma_sub(v - 2);
@@ -558,7 +632,20 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     // immediate (about 20 vector and 12 scalar instructions less per iteration; headline -2 %).  The
     // bf16 kernel with BM = 256 has no registers for the longer live ranges (it would spill) and
     // keeps the rolled loop.
-    if (W8 || PF == 2) {
+    if (PAIR8) {
+        // stage kt+1 belongs to pair (kt+1)/2, whose register set alternates: by four, every index is a literal
+        int kt = 0;
+        for (; kt + 4 <= nk; kt += 4) {
+            iteration(kt, 0, 0, 0);
+            iteration(kt + 1, 1, 1, 1);
+            iteration(kt + 2, 0, 0, 1);
+            iteration(kt + 3, 1, 1, 0);
+        }
+        if (kt < nk) {                       // (an even number of stages: fp8 scales come per 128 k)
+            iteration(kt, 0, 0, 0);
+            iteration(kt + 1, 1, 1, 1);
+        }
+    } else if (W8 || PF == 2) {
         int kt = 0;
         for (; kt + 2 <= nk; kt += 2) {
             iteration(kt, 0, 0);
