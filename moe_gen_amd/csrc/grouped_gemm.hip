@@ -93,9 +93,10 @@ typedef const __attribute__((address_space(1))) float* gptr_f32;
 typedef const __attribute__((address_space(1))) int32_t* gptr_i32;
 
 __device__ __forceinline__ u32x4 gload16(const void* p) { return *(gptr_u32x4)(uintptr_t)p; }
-// Weights under 128- and 64-row tiles are streamed: a tile of them is used by one or two workgroups
-// and never again in the launch, so those loads are non-temporal (Mixtral-8x22B, 256 tokens: down
-// projection 0.325 -> 0.302 ms).  Under 256-row tiles the panels are shared through L2 and stay plain.
+// Weights under the one-workgroup-per-tile kernel are streamed: a tile of them is used by one workgroup (two
+// or more for an expert above 256 rows) and never again in the launch, so those loads are non-temporal
+// (Mixtral-8x22B, 256 tokens: down projection 0.325 -> 0.302 ms).  In the persistent kernel the panels are
+// shared through L2 and stay plain.
 template <bool STREAM>
 __device__ __forceinline__ u32x4 gload16_w(const void* p) {
     return STREAM ? __builtin_nontemporal_load((gptr_u32x4)(uintptr_t)p) : *(gptr_u32x4)(uintptr_t)p;
@@ -160,14 +161,14 @@ __device__ __forceinline__ u32x2 epilogue_pack(const f32x4& a, const f32x4& up) 
     return u32x2{pack_bf16(a[0], a[1]), pack_bf16(a[2], a[3])};
 }
 
-// Exclusive scan of the experts' M-tile counts, ceil(count / BM), by the whole workgroup: s_pref[e] = number of
+// Exclusive scan of the experts' M-tile counts, tiles_of(count), by the whole workgroup: s_pref[e] = number of
 // M tiles in front of expert e (the caller adds s_pref[E] if it needs it).  Returns the total; the thread that
 // handled expert tid in the LAST pass keeps that expert's prefix, tile count and row range in `mine`
 // (experts beyond NT take further passes), and per_expert(e, first_row, end_row) runs once per expert.
 struct ExpertOfThread { int start, mt, o0, o1; };
-template <int NT, int BM, typename F>
+template <int NT, typename T, typename F>
 __device__ __forceinline__ int mtile_prefix_scan(const GemmArgs& g, int tid, int* s_pref, int* s_wtot,
-                                                 ExpertOfThread& mine, F per_expert) {
+                                                 ExpertOfThread& mine, T tiles_of, F per_expert) {
     const int lane = tid & 63, wave = tid >> 6;
     int run = 0;
     mine = ExpertOfThread{0, 0, 0, 0};
@@ -177,7 +178,7 @@ __device__ __forceinline__ int mtile_prefix_scan(const GemmArgs& g, int tid, int
         if (e < g.E) {
             mine.o0 = g.offsets[e];
             mine.o1 = g.offsets[e + 1];
-            mt = (mine.o1 - mine.o0 + BM - 1) / BM;
+            mt = tiles_of(mine.o1 - mine.o0);
             per_expert(e, mine.o0, mine.o1);
         }
         int inc = mt;
@@ -260,15 +261,19 @@ __device__ __forceinline__ void store_wave_outputs(const f32x4 (&acc)[2 * MT][TN
     }
 }
 
-// MT: 32-row units per wave along M (workgroup rows BM = 64*MT, 2 waves along M)
+// One tile of the one-workgroup-per-tile kernel: rows [row0, min(row0 + 64 MT, row_end)) of expert e times N tile n_tile.
+// MT: 32-row units per wave along M (tile rows BM = 64*MT, 2 waves along M)
 // WN: waves along N; 4 -> 8 waves of up to 128x64 outputs, two per SIMD; every wave interleaves
 //     its share of the load / dequantise / LDS-store work with its MFMAs, a piece per MFMA group
-template <int MT, int WN, bool SWIGLU, bool W8>
-__global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
+// smem0 / smem1: the two LDS stages (two separate arrays: stores into one stage and reads from the other provably
+//     do not alias, which lets the scheduler move them past each other)
+// STREAM: no other tile reads these weights (the expert has one M tile): non-temporal loads
+template <int MT, int WN, bool SWIGLU, bool W8, bool STREAM>
+__device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uint8_t* smem1, int e, int row0, int row_end,
+                                          int n_tile) {
     constexpr int NT = 128 * WN;                // threads
     constexpr int BM = 64 * MT;                 // rows per workgroup
     constexpr int A_STAGE = BM * ROW_B;         // bytes
-    constexpr int B_STAGE = BN_ROWS * ROW_B;
     constexpr int RA = NT / 8;                  // A rows covered by one pass of the workgroup
     constexpr int NA = BM / RA;                 // 16-byte A chunks per thread per stage
     constexpr int RB = W8 ? NT / 4 : NT / 8;    // B rows per pass (fp8 rows are 4 chunks of 16 weights)
@@ -276,68 +281,21 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     constexpr int NBLK = SWIGLU ? 128 : 256;    // output columns per workgroup
     constexpr int NJ = 8 / WN;                  // 32-row units of the weight tile per wave
     static_assert(NA >= 1 && NB >= 2, "tile/thread mismatch");
-    // two separate arrays: stores into one stage and reads from the other provably do not alias,
-    // which lets the scheduler move them past each other
-    __shared__ __attribute__((aligned(16))) uint8_t smem0[A_STAGE + B_STAGE];
-    __shared__ __attribute__((aligned(16))) uint8_t smem1[A_STAGE + B_STAGE];
-    __shared__ int s_pref[MAX_E + 1];
-    __shared__ int s_wtot[NT / 64];
-    __shared__ int s_sel[5];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave & 1, wn = (wave >> 1) % WN;
-
-    // ---- M-tile prefix over experts ----
-    ExpertOfThread mine;
-    const int run = mtile_prefix_scan<NT, BM>(g, tid, s_pref, s_wtot, mine, [](int, int, int) {});
-    const int total = run * g.n_tiles_n;
-
-    // ---- XCD-aware id: XCD x (= blockIdx % 8) owns tiles [x*per, (x+1)*per) ----
-    const int per = (total + 7) / 8;
-    const int slot = blockIdx.x >> 3;
-    const int v = (blockIdx.x & 7) * per + slot;
-    if (slot >= per || v >= total) return;
-    const int q = v / g.n_tiles_n;  // global M-tile number
-    // find e with prefix[e] <= q < prefix[e+1].  Up to NT experts every thread still holds its own
-    // expert's prefix, tile count and row range: the one that owns q publishes them (one barrier,
-    // no search, no second trip to memory for the offsets).  More experts: binary search in LDS.
-    if (g.E <= NT) {
-        if (tid < g.E && mine.start <= q && q < mine.start + mine.mt) {
-            s_sel[0] = tid; s_sel[1] = mine.start; s_sel[2] = mine.mt; s_sel[3] = mine.o0; s_sel[4] = mine.o1;
-        }
-        __syncthreads();
-    } else {
-        if (tid == 0) s_pref[g.E] = run;
-        __syncthreads();
-        int lo = 0, hi = g.E;
-        while (hi - lo > 1) {
-            int mid = (lo + hi) >> 1;
-            if (s_pref[mid] <= q) lo = mid; else hi = mid;
-        }
-        if (tid == 0) {
-            s_sel[0] = lo; s_sel[1] = s_pref[lo]; s_sel[2] = s_pref[lo + 1] - s_pref[lo];
-            s_sel[3] = g.offsets[lo]; s_sel[4] = g.offsets[lo + 1];
-        }
-        __syncthreads();
-    }
-    const int e = uni(s_sel[0]);
-    const int pe = uni(s_sel[1]);
-    const int mt_e = uni(s_sel[2]);
-    int m_tile, n_tile;
-    tile_in_expert(v - pe * g.n_tiles_n, mt_e, g.n_tiles_n, m_tile, n_tile);
-    const int row0 = uni(s_sel[3]) + m_tile * BM;
-    const int row_end = uni(s_sel[4]);
     const int n0 = n_tile * NBLK;
     const int K = g.K, N = g.N;
     const int nk = K / BK;
-    // Tiles below 256 rows mostly stream weights, and neighbouring workgroups start together: were they all to walk k
-    // from 0, every request in flight on the chip would carry the same low address bits (rows are K elements apart)
-    // and crowd a few memory channels.  N tile t walks k from stage t instead (mod nk; a dot product does not care
-    // where it starts, and a column's order depends on nothing but its position): Mixtral-8x22B, 256 tokens, down
-    // projection 0.302 -> 0.273 ms, gate/up 0.640 -> 0.620 ms.
-    // fp8 weights under these tiles are fetched 128 k at a time (see PAIR8 below): pairs of stages stay together
+    // These tiles mostly stream weights, and neighbouring workgroups start together: were they all to walk k from 0,
+    // every request in flight on the chip would carry the same low address bits (rows are K elements apart) and
+    // crowd a few memory channels.  N tile t walks k from stage t instead (mod nk; a dot product does not care
+    // where it starts, and a column's order depends on nothing but its position, whatever the tile height):
+    // Mixtral-8x22B, 256 tokens, down projection 0.302 -> 0.273 ms, gate/up 0.640 -> 0.620 ms.
+    // fp8 weights under tiles below 256 rows are fetched 128 k at a time (see PAIR8 below): pairs of stages stay
+    // together, so fp8 tiles start at stage 2 t
     constexpr bool PAIR8 = W8 && MT < 4;
-    const int rot = MT < 4 ? (PAIR8 ? (2 * n_tile) % nk : n_tile % nk) : 0;
+    const int rot = W8 ? (2 * n_tile) % nk : n_tile % nk;
     auto stage_at = [&](int kt) { const int kp = kt + rot; return kp >= nk ? kp - nk : kp; };
 
     // ---- per-thread load coordinates ----
@@ -422,7 +380,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
         int pr = min(pr_pipe, npair - 1) + prot;
         pr = pr >= npair ? pr - npair : pr;
         const uint8_t* m = (SWIGLU && i >= 2) ? bmat1 : bmat0;
-        rp[ps][i] = gload16_w<true>(past ? (const uint8_t*)g.a : m + (size_t)p_n[i] * K + (size_t)pr * 128 + ((tid & 7) << 4));
+        rp[ps][i] = gload16_w<STREAM>(past ? (const uint8_t*)g.a : m + (size_t)p_n[i] * K + (size_t)pr * 128 + ((tid & 7) << 4));
         if (i == 1) rps[ps][0] = sc0[srow0 + pr];
         if (i == 3) rps[ps][1] = sc1[srow1 + pr];
     };
@@ -450,7 +408,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
 #pragma unroll
         for (int i = 0; i < NB; ++i) {
             const uint8_t* m = (SWIGLU && i >= NB / 2) ? bmat1 : bmat0;  // rows >= 128 of the B tile are the up matrix
-            rb[set][i] = gload16_w<(MT < 4)>(m + ((size_t)b_n[i] * K + kofs) * EB + bcol_b);
+            rb[set][i] = gload16_w<STREAM>(m + ((size_t)b_n[i] * K + kofs) * EB + bcol_b);
         }
         if (W8) {
             rs[set][0] = sc0[srow0 + (kt >> 1)];
@@ -582,7 +540,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
         const size_t kofs = (size_t)kn * BK;
         // past the end nobody reads what is loaded: streamed weights would come from HBM once more
         // (PF + 1 stages per tile), so those loads take the first 16 bytes of the activations instead
-        const bool past = MT < 4 && kt + 1 + PF >= nk;
+        const bool past = kt + 1 + PF >= nk;
         if (i < NA) {
             *reinterpret_cast<u32x4*>(As + a_lds + i * RA * ROW_B) = ra[set][i];
             ra[set][i] = gload16(g.a + (size_t)a_src[i] * K + kofs + lchunk * 8);
@@ -603,7 +561,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
             // the first 8 weights go to b_lds[0], the second 8 to b_lds[1]; swapped rows the other way round
             *reinterpret_cast<u32x4*>(Bs + ((half ^ (b_swap ? 1 : 0)) ? b_lds[1] : b_lds[0]) + b * RB * ROW_B) = o;
             if (half == 1) {
-                rb[set][b] = gload16_w<(MT < 4)>(past ? (const uint8_t*)g.a : m + ((size_t)b_n[b] * K + kofs) * EB + bcol_b);
+                rb[set][b] = gload16_w<STREAM>(past ? (const uint8_t*)g.a : m + ((size_t)b_n[b] * K + kofs) * EB + bcol_b);
                 if (b / (NB / 2) == 0) rs[set][0] = sc0[srow0 + (kn >> 1)];
                 else rs[set][1] = sc1[srow1 + (kn >> 1)];
             }
@@ -611,7 +569,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
             const int b = i - NA;
             const uint8_t* m = (SWIGLU && b >= NB / 2) ? bmat1 : bmat0;
             *reinterpret_cast<u32x4*>(Bs + b_lds[0] + b * RB * ROW_B) = rb[set][b];
-            rb[set][b] = gload16_w<(MT < 4)>(past ? (const uint8_t*)g.a : m + ((size_t)b_n[b] * K + kofs) * EB + bcol_b);
+            rb[set][b] = gload16_w<STREAM>(past ? (const uint8_t*)g.a : m + ((size_t)b_n[b] * K + kofs) * EB + bcol_b);
         }
     };
     constexpr int NG = NU;                        // one group of MFMAs per slot
@@ -675,7 +633,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
         mfma_sub(NU - 1, part);
     };
     // (both forms pass the same barriers, so the waves of a workgroup may differ in theirs)
-    if (MT < 4 && !live[TM - 1]) k_loop(std::true_type{});
+    if (!live[TM - 1]) k_loop(std::true_type{});
     else k_loop(std::false_type{});
 
     // ---- epilogue ----
@@ -686,6 +644,71 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     const int ncol0 = n0 + wn * CW;
     store_wave_outputs<MT, TN, SWIGLU, 32 * MT, false>(acc, ep, lane, g.c + (size_t)(row0 + wm * 32 * MT) * N + ncol0, N,
                                                        min(BM, row_end - row0) - wm * 32 * MT, N - ncol0);
+}
+
+// M tiles of an expert with `count` rows in the one-workgroup-per-tile kernel: one tile of 64 rows if that holds
+// them all, else tiles of 128.  The height follows the EXPERT, not the launch: a tile taller than its expert
+// stages and multiplies rows that do not exist, and an expert cut into several tiles reads its weights once per
+// tile.  The tiles of such an expert (the hot one of a skewed decode batch) run side by side on one XCD and take
+// the weights with plain loads, so that all but the first read of a line come out of that XCD's L2.
+__device__ __forceinline__ int tiles_of(int count) { return count <= 64 ? (count > 0 ? 1 : 0) : (count + 127) >> 7; }
+
+// One workgroup per (M tile, N tile); serves what the persistent kernel does not take (few rows per expert, odd K).
+template <int WN, bool SWIGLU, bool W8>
+__global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
+    constexpr int NT = 128 * WN;
+    constexpr int STAGE_MAX = (128 + BN_ROWS) * ROW_B;   // a stage of the tallest tile
+    __shared__ __attribute__((aligned(16))) uint8_t smem0[STAGE_MAX];
+    __shared__ __attribute__((aligned(16))) uint8_t smem1[STAGE_MAX];
+    __shared__ int s_pref[MAX_E + 1];
+    __shared__ int s_wtot[NT / 64];
+    __shared__ int s_sel[5];
+    const int tid = threadIdx.x;
+
+    // ---- M-tile prefix over experts ----
+    ExpertOfThread mine;
+    const int run = mtile_prefix_scan<NT>(g, tid, s_pref, s_wtot, mine, [](int c) { return tiles_of(c); }, [](int, int, int) {});
+    const int total = run * g.n_tiles_n;
+
+    // ---- XCD-aware id: groups of 4 consecutive tiles (the M tiles of one N tile first) go round-robin to the XCDs
+    // (workgroup ids are dealt to the XCDs one by one).  The tiles of a multi-tile expert that read the same
+    // weights then share them through one XCD's L2, and dealing small groups round keeps the XCDs even whatever
+    // the number of tiles and however much one expert's tiles cost more than another's ----
+    const int slot = blockIdx.x >> 3;
+    const int v = (((slot >> 2) << 3) + (blockIdx.x & 7)) * 4 + (slot & 3);
+    if (v >= total) return;
+    const int q = v / g.n_tiles_n;  // global M-tile number
+    // find e with prefix[e] <= q < prefix[e+1].  Up to NT experts every thread still holds its own
+    // expert's prefix, tile count and row range: the one that owns q publishes them (one barrier,
+    // no search, no second trip to memory for the offsets).  More experts: binary search in LDS.
+    if (g.E <= NT) {
+        if (tid < g.E && mine.start <= q && q < mine.start + mine.mt) {
+            s_sel[0] = tid; s_sel[1] = mine.start; s_sel[2] = mine.mt; s_sel[3] = mine.o0; s_sel[4] = mine.o1;
+        }
+        __syncthreads();
+    } else {
+        if (tid == 0) s_pref[g.E] = run;
+        __syncthreads();
+        int lo = 0, hi = g.E;
+        while (hi - lo > 1) {
+            int mid = (lo + hi) >> 1;
+            if (s_pref[mid] <= q) lo = mid; else hi = mid;
+        }
+        if (tid == 0) {
+            s_sel[0] = lo; s_sel[1] = s_pref[lo]; s_sel[2] = s_pref[lo + 1] - s_pref[lo];
+            s_sel[3] = g.offsets[lo]; s_sel[4] = g.offsets[lo + 1];
+        }
+        __syncthreads();
+    }
+    const int e = uni(s_sel[0]);
+    const int pe = uni(s_sel[1]);
+    const int mt_e = uni(s_sel[2]);
+    const int first_row = uni(s_sel[3]), row_end = uni(s_sel[4]);
+    int m_tile, n_tile;
+    tile_in_expert(v - pe * g.n_tiles_n, mt_e, g.n_tiles_n, m_tile, n_tile);
+    if (row_end - first_row <= 64) gemm_tile<1, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
+    else if (mt_e == 1) gemm_tile<2, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
+    else gemm_tile<2, WN, SWIGLU, W8, false>(g, smem0, smem1, e, first_row + m_tile * 128, row_end, n_tile);
 }
 
 // lane id produced where it is used: the compiler cannot hoist it (and everything derived from it)
@@ -749,7 +772,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
 
     // M-tile prefix over experts; the experts' row offsets and matrix pointers go to LDS tables on the way
     ExpertOfThread mine;
-    const int run = mtile_prefix_scan<NT, BM>(g, tid, s_pref, s_wtot, mine, [&](int e, int o0, int o1) {
+    const int run = mtile_prefix_scan<NT>(g, tid, s_pref, s_wtot, mine, [](int c) { return (c + BM - 1) / BM; }, [&](int e, int o0, int o1) {
         s_off[e] = o0;
         if (e == g.E - 1) s_off[g.E] = o1;
         s_ptr[0][e] = (unsigned long long)(uintptr_t)g.b0[e];
@@ -1004,12 +1027,11 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
     }
 }
 
-template <int MT, int WN, bool SWIGLU, bool W8>
-int launch_one(const GemmArgs& g, int n_rows, hipStream_t st) {
-    constexpr int BM = 64 * MT;
-    auto kern = grouped_gemm_kernel<MT, WN, SWIGLU, W8>;
-    const long max_mtiles = (long)n_rows / BM + g.E;  // sum_e ceil(c_e/BM) <= n_rows/BM + E
-    const long grid = ((max_mtiles * g.n_tiles_n + 7) / 8) * 8;
+template <int WN, bool SWIGLU, bool W8>
+int launch_tiles(const GemmArgs& g, int n_rows, hipStream_t st) {
+    auto kern = grouped_gemm_kernel<WN, SWIGLU, W8>;
+    const long max_mtiles = (long)n_rows / 128 + g.E;  // sum_e tiles_of(c_e) <= sum_e (c_e / 128 + 1)
+    const long grid = ((max_mtiles * g.n_tiles_n + 31) / 32) * 32;   // whole rounds of 8 groups of 4 tiles
     if (grid > 0x7fffffffL) {
         set_error("grouped gemm: %ld workgroups exceed the grid limit", grid);
         return MOE_ERR_INVALID;
@@ -1050,13 +1072,7 @@ int launch_mt(const GemmArgs& g, int n_rows, hipStream_t st) {
     // one), keeps per-expert tables for up to 512 experts and addresses gathered rows with 32-bit offsets
     const bool fits = !g.row_map || g.a_bytes < (1ull << 32);
     if (mean >= 192 && g.K % 128 == 0 && g.E <= 512 && fits && cu_count() >= 8) return launch_persistent<SWIGLU, W8>(g, n_rows, st);
-    // The counts themselves live on the device; only their mean is known here.  Routing is
-    // uneven, so around a mean of 64 rows some experts exceed 64 and would stream their weights
-    // once per 64-row tile: 128-row tiles from a mean of 48 (Mixtral-8x22B decode, 256 tokens:
-    // down projection 0.50 -> 0.32 ms; with perfectly even counts the larger tile costs ~4 %).
-    if (mean >= 192) return launch_one<4, 4, SWIGLU, W8>(g, n_rows, st);
-    if (mean >= 48) return launch_one<2, 4, SWIGLU, W8>(g, n_rows, st);
-    return launch_one<1, 4, SWIGLU, W8>(g, n_rows, st);
+    return launch_tiles<4, SWIGLU, W8>(g, n_rows, st);
 }
 
 template <bool W8>

@@ -74,7 +74,7 @@ def run_case(E, h, I, counts, fp8, seed, use_row_map=False):
     (4, 256, 384, [0, 1, 255, 257]),
     (8, 512, 256, [5, 0, 130, 64, 0, 0, 700, 31]),
     (3, 1024, 640, [1000, 3, 500]),
-    (8, 256, 256, [3, 0, 40, 17, 0, 1, 64, 9]),        # mean < 48 rows per expert: the 64-row tile
+    (8, 256, 256, [3, 0, 40, 17, 0, 1, 64, 9]),        # every expert under a 64-row tile
     (6, 384, 128, [70, 2, 0, 33, 1, 5]),
     (2, 128, 128, [1, 0]),
     (4, 384, 256, [300, 500, 0, 260]),                 # 256-row tiles, ragged last N tile of the down projection
@@ -90,9 +90,9 @@ def test_grouped_swiglu_vs_oracle(fp8, E, h, I, counts):
 
 
 @pytest.mark.parametrize("E,h,I,counts", [
-    (1, 192, 320, [300]),            # 256-row tile
-    (2, 192, 320, [100, 30]),        # 128-row tile
-    (4, 320, 192, [5, 9, 0, 20]),    # 64-row tile
+    (1, 192, 320, [300]),            # three 128-row tiles
+    (2, 192, 320, [100, 30]),        # a 128-row tile and a 64-row tile
+    (4, 320, 192, [5, 9, 0, 20]),    # 64-row tiles
     (1, 64, 64, [70]),               # a single k-stage
     (4, 384, 320, [300, 500, 0, 260]),   # gate/up: even stage count, ragged last N tile; down: 5 stages
 ])
@@ -105,11 +105,42 @@ def test_grouped_odd_stage_counts(E, h, I, counts):
 
 
 @pytest.mark.parametrize("fp8", [False, True])
+def test_tile_height_follows_the_expert(fp8):
+    """One launch of the one-workgroup-per-tile kernel (mean rows per expert below 192) with experts on both
+    sides of every tile-height boundary: a 64-row tile up to 64 rows, one 128-row tile up to 128, several
+    128-row tiles above (those read their weights with plain loads).  Against the oracle, and an expert's rows
+    bit-for-bit against a launch that holds this expert alone."""
+    from moe_gen_amd import ops
+    E, h, I = 10, 512, 384
+    counts = [3, 64, 65, 128, 129, 300, 0, 17, 257, 1]
+    print(f"tile heights fp8={fp8} counts={counts}", flush=True)
+    y, ref32, refr = run_case(E, h, I, counts, fp8, seed=61, use_row_map=True)
+    assert np.isfinite(y).all() and rel_max(y, ref32) <= TOL and rel_max(y, refr) <= TOL
+    # the same experts one at a time (run_case draws x and the weights from the seed alone)
+    offsets = np.concatenate([[0], np.cumsum(counts)])
+    mats = make_experts(E, h, I, fp8, 62)
+    g = torch.Generator().manual_seed(61)
+    x = torch.randn(int(offsets[-1]), h, generator=g).to(torch.bfloat16)
+    dev = lambda m: tuple(t.cuda() for t in m) if isinstance(m, tuple) else m.cuda()
+    for e in (1, 2, 4):                                  # 64, 65 and 129 rows: alone they stay below 192 rows too
+        one = [dev(m) for m in mats[e]]
+        if fp8:
+            ptrs = ops.expert_pointers([one[0][0]], [one[1][0]], [one[2][0]], [one[0][1]], [one[1][1]], [one[2][1]])
+        else:
+            ptrs = ops.expert_pointers([one[0]], [one[1]], [one[2]])
+        a, b = int(offsets[e]), int(offsets[e + 1])
+        ye = ops.grouped_swiglu(x[a:b].cuda(), None, ptrs, torch.tensor([0, b - a], dtype=torch.int32, device="cuda"), b - a)
+        torch.cuda.synchronize()
+        assert np.array_equal(O.bf16_to_f32(bits(ye)), y[a:b]), f"expert {e} differs from its launch alone"
+
+
+@pytest.mark.parametrize("fp8", [False, True])
 @pytest.mark.parametrize("E,mean", [(700, 3), (1024, 2), (600, 200), (400, 200)])
 def test_grouped_many_experts(fp8, E, mean):
     """More experts than threads in a workgroup (the M-tile prefix scan takes two passes), up to the
-    maximum of 1024, with empty experts sprinkled in; the last two cases take the 256-row tile (400
-    experts: the persistent kernel with its per-expert tables in LDS; 600: one workgroup per tile)."""
+    maximum of 1024, with empty experts sprinkled in; the last two cases have about 200 rows per expert (400
+    experts: the persistent kernel with its per-expert tables in LDS; 600: one workgroup per tile, two
+    128-row tiles for most experts)."""
     print(f"grouped many experts fp8={fp8} E={E} mean={mean}", flush=True)
     rng = np.random.default_rng(E)
     counts = rng.poisson(mean, E)
@@ -254,8 +285,8 @@ def test_persistent_kernel_corner_shapes(fp8, E, h, I, counts):
 @pytest.mark.parametrize("n_src,n", [(300, 600), (60, 120)])
 def test_row_map_may_repeat_rows(n_src, n):
     """Several sorted rows may name the same source row (a token routed to k experts).  Both launches of a case
-    run the same tile kernel (256-row tiles / 128-row tiles): kernels of different tile heights walk k from
-    different stages and may differ in the last bit."""
+    run the same kernel (the persistent kernel / one workgroup per tile): the two walk k from different stages
+    and may differ in the last bit."""
     from moe_gen_amd import ops
     h, I = 256, 256
     ws, ptrs = _one_expert(h, I, 51)
