@@ -119,3 +119,42 @@ def test_block_edge_shapes(name):
     torch.cuda.synchronize()
     assert int((blk.last_counts > 0).sum()) == w.k and int(blk.last_counts.max()) == 64
     assert torch.equal(out, full[:, :1].expand_as(out))
+
+
+@pytest.mark.parametrize("name", ["mixtral_8x22b_decode", "deepseek_v2_lite", "deepseek_v3_w8a16"])
+def test_block_forward_can_be_captured_in_a_graph(name):
+    """The block's forward with resident weights launches kernels and nothing else (no host read, no memset, no
+    allocation outside torch's), so a decode loop may capture it in a HIP graph.  Replayed three times with eager
+    forwards and synchronisations in between, then on a new input: every replay bit-for-bit the eager result."""
+    from moe_gen_amd import synthetic
+    w = small(name)
+    print(f"graph capture {name}", flush=True)
+    blk = synthetic.build_block(w, device="cuda", gen_device="cpu")
+    first = lambda o: o[0] if isinstance(o, tuple) else o
+    x = synthetic.hidden_states(w, "cuda")
+    y_ref = first(blk(x)).clone()
+    torch.cuda.synchronize()
+    x_static = x.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            blk(x_static)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y_static = first(blk(x_static))
+    torch.cuda.synchronize()
+    for it in range(3):
+        y_static.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_static, y_ref), f"replay {it} differs from the eager forward"
+        assert torch.equal(first(blk(x)), y_ref)         # the program's own eager work between the replays
+        torch.cuda.synchronize()
+    x2 = x.flip(0).contiguous()
+    y2 = first(blk(x2)).clone()
+    x_static.copy_(x2)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(y_static, y2), "replay on a new input differs from the eager forward"
