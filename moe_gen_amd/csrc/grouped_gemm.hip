@@ -465,7 +465,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
     // two small buffers.  Slot v of an iteration issues the MFMAs of sub-phase v-2 (the last two
     // sub-phases of a stage run in the first two slots of the next iteration, across the workgroup
     // barrier) and then requests the fragments of sub-phase v, whose buffer those MFMAs just freed.
-    constexpr int TQ = (MT >= 2) ? MT / 2 : 1;    // token tiles per part
+    constexpr int TQ = MT == 3 ? 3 : (MT >= 2) ? MT / 2 : 1;    // token tiles per part (the parts per k-step, 2 MT / TQ, must divide the 4 weight tiles)
     constexpr int NP = TM / TQ;                   // parts per k-step
     constexpr int NU = 2 * NP;                    // sub-phases per stage
     bf16x8 wfr[2][TN], tq[2][TQ];
@@ -646,18 +646,21 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
                                                        min(BM, row_end - row0) - wm * 32 * MT, N - ncol0);
 }
 
-// M tiles of an expert with `count` rows in the one-workgroup-per-tile kernel: one tile of 64 rows if that holds
-// them all, else tiles of 128.  The height follows the EXPERT, not the launch: a tile taller than its expert
-// stages and multiplies rows that do not exist, and an expert cut into several tiles reads its weights once per
-// tile.  The tiles of such an expert (the hot one of a skewed decode batch) run side by side on one XCD and take
-// the weights with plain loads, so that all but the first read of a line come out of that XCD's L2.
-__device__ __forceinline__ int tiles_of(int count) { return count <= 64 ? (count > 0 ? 1 : 0) : (count + 127) >> 7; }
+// M tiles of an expert with `count` rows in the one-workgroup-per-tile kernel: one tile of 64, 128 or (bf16 weights)
+// 192 rows if that holds them all, else tiles of 128.  The height follows the EXPERT, not the launch: a tile taller
+// than its expert stages and multiplies rows that do not exist, and an expert cut into several tiles reads its
+// weights once per tile and adds workgroups (the hot expert of a skewed decode batch: 9 x 128 tiles are 4.5 rounds
+// of 256 CUs and cost 5).  The tiles of an expert that is cut (above 192 rows; above 128 with fp8 weights, where the
+// 192-row body does not fit the registers) run side by side on one XCD and take the weights with plain loads, so
+// that all but the first read of a line come out of that XCD's L2.
+template <int SINGLE>   // rows that one tile may hold
+__device__ __forceinline__ int tiles_of(int count) { return count <= SINGLE ? (count > 0 ? 1 : 0) : (count + 127) >> 7; }
 
 // One workgroup per (M tile, N tile); serves what the persistent kernel does not take (few rows per expert, odd K).
 template <int WN, bool SWIGLU, bool W8>
 __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     constexpr int NT = 128 * WN;
-    constexpr int STAGE_MAX = (128 + BN_ROWS) * ROW_B;   // a stage of the tallest tile
+    constexpr int STAGE_MAX = ((W8 ? 128 : 192) + BN_ROWS) * ROW_B;   // a stage of the tallest tile
     __shared__ __attribute__((aligned(16))) uint8_t smem0[STAGE_MAX];
     __shared__ __attribute__((aligned(16))) uint8_t smem1[STAGE_MAX];
     __shared__ int s_pref[MAX_E + 1];
@@ -667,7 +670,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
 
     // ---- M-tile prefix over experts ----
     ExpertOfThread mine;
-    const int run = mtile_prefix_scan<NT>(g, tid, s_pref, s_wtot, mine, [](int c) { return tiles_of(c); }, [](int, int, int) {});
+    const int run = mtile_prefix_scan<NT>(g, tid, s_pref, s_wtot, mine, [](int c) { return tiles_of<(W8 ? 128 : 192)>(c); }, [](int, int, int) {});
     const int total = run * g.n_tiles_n;
 
     // ---- XCD-aware id: groups of 4 consecutive tiles (the M tiles of one N tile first) go round-robin to the XCDs
@@ -707,7 +710,8 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     int m_tile, n_tile;
     tile_in_expert(v - pe * g.n_tiles_n, mt_e, g.n_tiles_n, m_tile, n_tile);
     if (row_end - first_row <= 64) gemm_tile<1, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
-    else if (mt_e == 1) gemm_tile<2, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
+    else if (row_end - first_row <= 128) gemm_tile<2, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
+    else if (!W8 && mt_e == 1) gemm_tile<3, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
     else gemm_tile<2, WN, SWIGLU, W8, false>(g, smem0, smem1, e, first_row + m_tile * 128, row_end, n_tile);
 }
 
