@@ -84,7 +84,9 @@ def cpu_baseline(w, blk, n_sample: int, passes: int = 3):
 def staged_run(w, blk, x, steps: int, routing_aware: bool = False, pool: int = 0):
     """Second figure: the same block with every expert matrix in pinned host memory, delivered by
     the stager (cyclic prefetch on the copy stream, event hand-off) into a pool of `pool` slots while
-    earlier experts are multiplied.  Two layers' worth of modules alternate, as in a model.
+    earlier experts are multiplied.  Three layers' worth of modules take turns, as in a model (with two, the
+    layer before the current one is also the next one, and the engine's rule that drops what is left of the
+    previous layer would throw away what it has just prefetched whenever the pool holds two layers).
     routing_aware: copy only the experts that received tokens, busiest first, once the per-expert
     counts are known (fewer bytes, but the copies cannot start before the router has run)."""
     import time as _t
@@ -105,7 +107,7 @@ def staged_run(w, blk, x, steps: int, routing_aware: bool = False, pool: int = 0
         n_slots["shared_expert"] = 2
     st = Stager(shapes, n_slots, device="cuda:0", model_type={"v3": "deepseek_v3", "v2": "deepseek_v2"}.get(w.family, "mixtral"),
                 num_hidden_layers=64, num_local_experts=E)
-    layers = (10, 11)
+    layers = (10, 11, 12)
     if routing_aware:
         st.set_policy("routed_expert", "on_demand")
 
@@ -132,7 +134,7 @@ def staged_run(w, blk, x, steps: int, routing_aware: bool = False, pool: int = 0
     import torch.nn as nn
 
     def step(i):
-        ex, sh = staged[layers[i % 2]]
+        ex, sh = staged[layers[i % len(layers)]]
         blk.experts = nn.ModuleList(ex)
         if has_shared:
             blk.shared_experts = sh
@@ -140,7 +142,8 @@ def staged_run(w, blk, x, steps: int, routing_aware: bool = False, pool: int = 0
 
     blk.routing_aware_staging = routing_aware
     st.pump()
-    step(0); step(1)
+    for i in range(len(layers)):
+        step(i)
     torch.cuda.synchronize()
     c0, b0 = st.stats()
     t0 = _t.perf_counter()
