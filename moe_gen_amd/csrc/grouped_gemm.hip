@@ -12,19 +12,22 @@
 // w = bf16(f32(q) * scale[i/128, j/128]).
 //
 // Work decomposition.  Sorted rows of expert e are [offsets[e], offsets[e+1]).  Each
-// expert is cut into M tiles of BM rows (the last one partial); an M tile times an N tile
-// of the weight matrix is one workgroup.  Every workgroup rebuilds the (tiny) M-tile
-// prefix over experts in LDS from offsets[], so the launch needs neither a host sync nor
-// a tile table: grid = upper bound on the tile count, surplus workgroups exit at once.
-// Workgroup ids are dealt round-robin to the 8 XCDs by the hardware; the id is remapped
-// so that each XCD owns a contiguous range of tiles (same expert, neighbouring M/N
-// tiles), which is what makes its private L2 hold the A and B panels that are re-read.
-// For 256-row tiles (grouped_gemm_persistent_kernel) the launch has one workgroup per CU
-// instead, groups of 32 consecutive tiles go round-robin to the XCDs, and a workgroup's k
-// pipeline runs on from one of its tiles into the next.
+// expert is cut into M tiles (the last one partial); an M tile times an N tile of the
+// weight matrix is one unit of work.  Every workgroup rebuilds the (tiny) M-tile prefix
+// over experts in LDS from offsets[], so a launch needs neither a host sync nor a tile table.
+// Two kernels:
+//  * grouped_gemm_persistent_kernel (from a mean of 192 rows per expert): 256-row tiles, one
+//    workgroup per CU, groups of 32 consecutive tiles go round-robin to the XCDs (workgroup
+//    ids are dealt to the 8 XCDs one by one by the hardware; the tiles of a group share their
+//    A and B panels through that XCD's L2), and a workgroup's k pipeline runs on from one of
+//    its tiles into the next.
+//  * grouped_gemm_kernel (fewer rows per expert, a launch that mostly streams weights): one
+//    workgroup per tile, grid = upper bound on the tile count, surplus workgroups exit at once;
+//    the tile height (64, 128 or 192 rows) follows the expert, groups of 4 tiles go round-robin
+//    to the XCDs.
 //
-// Workgroup = 8 waves (2 along M, 4 along N), two per SIMD.  Per wave 2*MT x 4 MFMA tiles of
-// 16x16 (v_mfma_f32_16x16x32_bf16), i.e. up to 128x64 outputs and 128 fp32 accumulators.  On
+// Workgroup = 8 waves (2 along M, 4 along N), two per SIMD.  Per wave 2, 4, 6 or 8 x 4 MFMA tiles
+// of 16x16 (v_mfma_f32_16x16x32_bf16), i.e. up to 128x64 outputs and 128 fp32 accumulators.  On
 // real (non-zero) data this chip is power-limited under MFMA load; the 16x16x32 shape moves a
 // third less accumulator data per flop than 32x32x16 and sustains ~13 % more (1.95 vs 1.73
 // PFLOP/s in a registers-only loop with random operands), which is worth ~6 % here.
