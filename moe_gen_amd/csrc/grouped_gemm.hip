@@ -279,11 +279,11 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
     constexpr int A_STAGE = BM * ROW_B;         // bytes
     constexpr int RA = NT / 8;                  // A rows covered by one pass of the workgroup
     constexpr int NA = BM / RA;                 // 16-byte A chunks per thread per stage
-    constexpr int RB = W8 ? NT / 4 : NT / 8;    // B rows per pass (fp8 rows are 4 chunks of 16 weights)
-    constexpr int NB = BN_ROWS / RB;            // 16-byte global B chunks per thread per stage
+    constexpr int RB = NT / 8;                  // B rows per pass of the workgroup (8 lanes per 128-byte row)
+    constexpr int NB = BN_ROWS / RB;            // 16-byte global B chunks per thread per stage (fp8: per pair of stages)
     constexpr int NBLK = SWIGLU ? 128 : 256;    // output columns per workgroup
     constexpr int NJ = 8 / WN;                  // 32-row units of the weight tile per wave
-    static_assert(NA >= 1 && NB >= 2, "tile/thread mismatch");
+    static_assert(MT <= 3 && NA >= 1 && NB == 4, "tile/thread mismatch");
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave & 1, wn = (wave >> 1) % WN;
@@ -297,7 +297,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
     // Mixtral-8x22B, 256 tokens, down projection 0.302 -> 0.273 ms, gate/up 0.640 -> 0.620 ms.
     // fp8 weights under tiles below 256 rows are fetched 128 k at a time (see PAIR8 below): pairs of stages stay
     // together, so fp8 tiles start at stage 2 t
-    constexpr bool PAIR8 = W8 && MT < 4;
+    constexpr bool PAIR8 = W8;
     const int rot = W8 ? (2 * n_tile) % nk : n_tile % nk;
     auto stage_at = [&](int kt) { const int kp = kt + rot; return kp >= nk ? kp - nk : kp; };
 
@@ -315,9 +315,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
     const uint8_t* bmat1 = SWIGLU ? uni_ptr(g.b1[e]) : bmat0;
     gptr_f32 sc0 = W8 ? (gptr_f32)(uintptr_t)uni_ptr(g.s0[e]) : nullptr;
     gptr_f32 sc1 = (W8 && SWIGLU) ? (gptr_f32)(uintptr_t)uni_ptr(g.s1[e]) : sc0;
-    constexpr int EB = W8 ? 1 : 2;                        // bytes per weight element
-    const int brow = W8 ? (tid >> 2) : (tid >> 3);        // fp8 tiles: row tid/4 (+RB i), 16-byte chunk tid%4
-    const int bcol_b = W8 ? ((tid & 3) << 4) : ((tid & 7) << 4);  // byte offset inside the 64-element k slab
+    // weight rows: thread (row tid/8 + 64 i of the tile, 16-byte chunk tid%8 of a 128-byte piece of the row: one
+    // k-stage of bf16 weights, a pair of k-stages of fp8 weights)
+    const int brow = tid >> 3, bcol_b = (tid & 7) << 4;
     int b_n[NB];
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
@@ -325,19 +325,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
         int n = SWIGLU ? (n0 + (r & 127)) : (n0 + r);
         b_n[i] = min(n, N - 1);
     }
-    uint32_t b_lds[2];
-    // fp8: a thread owns chunks 2q and 2q+1 of its row; rows with bit 1 set store them in the
-    // opposite order so that the 16 lanes of one store instruction (4 rows x 4 chunks) spread
-    // over all banks
-    const bool b_swap = W8 && ((brow >> 1) & 1);
-    if (W8) {
-        int qd = tid & 3, sw = swz(brow), first = b_swap ? 1 : 0;
-        b_lds[0] = (uint32_t)(brow * ROW_B + (((2 * qd + first) ^ sw) << 4));
-        b_lds[1] = (uint32_t)(brow * ROW_B + (((2 * qd + 1 - first) ^ sw) << 4));
-    } else {
-        b_lds[0] = (uint32_t)(brow * ROW_B + (((tid & 7) ^ swz(brow)) << 4));
-        b_lds[1] = 0;
-    }
+    const uint32_t b_lds = (uint32_t)(brow * ROW_B + (((tid & 7) ^ swz(brow)) << 4));   // (bf16 weights)
     // block-scale rows (W8): first / second 128 rows of the B tile
     int srow0 = 0, srow1 = 0;
     const int KB = K >> 7;
@@ -352,7 +340,6 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
     // limits the HBM rate.
     constexpr int PF = (MT <= 2) ? 2 : 1;
     u32x4 ra[PF][NA], rb[PF][NB];
-    float rs[PF][2];
 
     // PAIR8.  A 64-k stage of fp8 weights is 64 bytes of a row, half a cache line: fetched stage by stage, every
     // row costs two half-line requests, and a CU can only keep so many requests in flight whatever their size
@@ -363,27 +350,19 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
     // store each, the unit of work of a data item): chunk 2 (c%4) + (c/4 ^ stage) of the stage's LDS row.  Two
     // register sets of pairs; a set is refilled while the second stage of its pair is stored, three
     // iterations before it is needed again.
-    const int prow = tid >> 3, pq = tid & 3, phb = (tid >> 2) & 1;
+    const int pq = tid & 3, phb = (tid >> 2) & 1;
     u32x4 rp[2][4];
     float rps[2][2];
-    int p_n[4];
     uint32_t p_lds[2];
-    if (PAIR8) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int r = prow + 64 * i;
-            p_n[i] = min(SWIGLU ? n0 + (r & 127) : n0 + r, N - 1);
-        }
-#pragma unroll
-        for (int st = 0; st < 2; ++st) p_lds[st] = (uint32_t)(prow * ROW_B + (((2 * pq + (phb ^ st)) ^ swz(prow)) << 4));
-    }
+    for (int st = 0; st < 2; ++st) p_lds[st] = (uint32_t)(brow * ROW_B + (((2 * pq + (phb ^ st)) ^ swz(brow)) << 4));
     const int npair = nk >> 1, prot = rot >> 1;
     auto pair_load = [&](int pr_pipe, int ps, int i) {      // chunk i of pair pr_pipe (pipeline order) into set ps
         const bool past = pr_pipe >= npair;                  // nobody reads it: not from the weights
         int pr = min(pr_pipe, npair - 1) + prot;
         pr = pr >= npair ? pr - npair : pr;
         const uint8_t* m = (SWIGLU && i >= 2) ? bmat1 : bmat0;
-        rp[ps][i] = gload16_w<STREAM>(past ? (const uint8_t*)g.a : m + (size_t)p_n[i] * K + (size_t)pr * 128 + ((tid & 7) << 4));
+        rp[ps][i] = gload16_w<STREAM>(past ? (const uint8_t*)g.a : m + (size_t)b_n[i] * K + (size_t)pr * 128 + bcol_b);
         if (i == 1) rps[ps][0] = sc0[srow0 + pr];
         if (i == 3) rps[ps][1] = sc1[srow1 + pr];
     };
@@ -400,7 +379,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
     };
     auto pair_store = [&](uint8_t* Bs, int ps, int i, int st) {   // the 8 weights of stage st of the pair -> LDS
         const u32x4 o = dequant8(rp[ps][i][2 * st], rp[ps][i][2 * st + 1], rps[ps][i >> 1]);
-        *reinterpret_cast<u32x4*>(Bs + p_lds[st] + i * 64 * ROW_B) = o;
+        *reinterpret_cast<u32x4*>(Bs + p_lds[st] + i * RB * ROW_B) = o;
     };
     auto gload = [&](int kt_pipe, int set) {
         const int kt = stage_at(kt_pipe);
@@ -411,11 +390,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
 #pragma unroll
         for (int i = 0; i < NB; ++i) {
             const uint8_t* m = (SWIGLU && i >= NB / 2) ? bmat1 : bmat0;  // rows >= 128 of the B tile are the up matrix
-            rb[set][i] = gload16_w<STREAM>(m + ((size_t)b_n[i] * K + kofs) * EB + bcol_b);
-        }
-        if (W8) {
-            rs[set][0] = sc0[srow0 + (kt >> 1)];
-            rs[set][1] = sc1[srow1 + (kt >> 1)];
+            rb[set][i] = gload16_w<STREAM>(m + ((size_t)b_n[i] * K + kofs) * 2 + bcol_b);
         }
     };
     auto lds_store = [&](uint8_t* As, int set) {
@@ -428,17 +403,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
                 pair_swap(0, i);
                 pair_store(Bs, 0, i, 0);
             }
-        } else if (W8) {
-#pragma unroll
-            for (int i = 0; i < NB; ++i) {
-                u32x4 l, h;
-                dequant16(rb[set][i], rs[set][i / (NB / 2)], l, h);
-                *reinterpret_cast<u32x4*>(Bs + b_lds[0] + i * RB * ROW_B) = b_swap ? h : l;
-                *reinterpret_cast<u32x4*>(Bs + b_lds[1] + i * RB * ROW_B) = b_swap ? l : h;
-            }
         } else {
 #pragma unroll
-            for (int i = 0; i < NB; ++i) *reinterpret_cast<u32x4*>(Bs + b_lds[0] + i * RB * ROW_B) = rb[set][i];
+            for (int i = 0; i < NB; ++i) *reinterpret_cast<u32x4*>(Bs + b_lds + i * RB * ROW_B) = rb[set][i];
         }
     };
 
@@ -534,8 +501,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
     // tile kt+1+PF.  The items are spread over the iteration, one per group of MFMAs, so LDS, the
     // vector-memory pipe and the matrix core see a steady mix instead of bursts; with exact load
     // waits each item stalls only until its own chunk (requested PF iterations earlier) is there.
-    constexpr int NBI = W8 ? 2 * NB : NB;      // (PAIR8: 4 rows, which is the same number)
-    constexpr int NI = NA + NBI;
+    constexpr int NI = NA + NB;
     // par = kt & 1 and ps, the register set of the pair that stage kt+1 belongs to, are literals at the call sites
     auto data_item = [&](int i, uint8_t* As, int kt, int set, int par, int ps) __attribute__((always_inline)) {
         uint8_t* Bs = As + A_STAGE;
@@ -556,23 +522,11 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
                 pair_store(Bs, ps, b, 1);
                 pair_load((kt >> 1) + 2, ps, b);
             }
-        } else if (W8) {
-            const int b = (i - NA) >> 1, half = (i - NA) & 1;
-            const uint8_t* m = (SWIGLU && b >= NB / 2) ? bmat1 : bmat0;
-            const float sc = rs[set][b / (NB / 2)];
-            const u32x4 o = dequant8(rb[set][b][2 * half], rb[set][b][2 * half + 1], sc);
-            // the first 8 weights go to b_lds[0], the second 8 to b_lds[1]; swapped rows the other way round
-            *reinterpret_cast<u32x4*>(Bs + ((half ^ (b_swap ? 1 : 0)) ? b_lds[1] : b_lds[0]) + b * RB * ROW_B) = o;
-            if (half == 1) {
-                rb[set][b] = gload16_w<STREAM>(past ? (const uint8_t*)g.a : m + ((size_t)b_n[b] * K + kofs) * EB + bcol_b);
-                if (b / (NB / 2) == 0) rs[set][0] = sc0[srow0 + (kn >> 1)];
-                else rs[set][1] = sc1[srow1 + (kn >> 1)];
-            }
         } else {
             const int b = i - NA;
             const uint8_t* m = (SWIGLU && b >= NB / 2) ? bmat1 : bmat0;
-            *reinterpret_cast<u32x4*>(Bs + b_lds[0] + b * RB * ROW_B) = rb[set][b];
-            rb[set][b] = gload16_w<STREAM>(past ? (const uint8_t*)g.a : m + ((size_t)b_n[b] * K + kofs) * EB + bcol_b);
+            *reinterpret_cast<u32x4*>(Bs + b_lds + b * RB * ROW_B) = rb[set][b];
+            rb[set][b] = gload16_w<STREAM>(past ? (const uint8_t*)g.a : m + ((size_t)b_n[b] * K + kofs) * 2 + bcol_b);
         }
     };
     constexpr int NG = NU;                        // one group of MFMAs per slot
@@ -586,8 +540,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
             // chunk are stored before its registers are refilled
 #pragma unroll
             for (int i0 = v * NI / NG; i0 < (v + 1) * NI / NG; ++i0) {
-                const int i = (W8 && NA == 4 && NI == 8) ? ((i0 & 1) ? NA + (i0 >> 1) : (i0 >> 1)) : i0;
-                data_item(i, wr, kt, set, par, ps);
+                data_item(i0, wr, kt, set, par, ps);
             }
             if (!W8) __builtin_amdgcn_sched_barrier(0);
             if (v >= 2) mfma_sub(v - 2, part);
