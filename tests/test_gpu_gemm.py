@@ -78,6 +78,7 @@ def run_case(E, h, I, counts, fp8, seed, use_row_map=False):
     (6, 384, 128, [70, 2, 0, 33, 1, 5]),
     (2, 128, 128, [1, 0]),
     (4, 384, 256, [300, 500, 0, 260]),                 # 256-row tiles, ragged last N tile of the down projection
+    (32, 256, 256, [3000] + [2] * 31),                 # one hot expert under a low mean: 24 tiles of 128 rows among 64-row tiles
 ])
 def test_grouped_swiglu_vs_oracle(fp8, E, h, I, counts):
     print(f"grouped fp8={fp8} E={E} h={h} I={I} counts={counts}", flush=True)
