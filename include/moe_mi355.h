@@ -138,7 +138,7 @@ int moe_dispatch_static(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k
  *   x         device bf16: rows of the sorted token matrix [n_rows, h]; or, when
  *             row_map != NULL, the unsorted matrix, row r being x[row_map[r]]
  *   x_rows    rows of x (>= 1).  It bounds the gather where rows are fetched through a buffer
- *             descriptor (from a mean of 192 rows per expert, x smaller than 4 GiB): a row_map entry outside [0, x_rows)
+ *             descriptor (experts on the persistent kernel, below; x smaller than 4 GiB): a row_map entry outside [0, x_rows)
  *             then reads zeros (or, once its byte offset wraps 32 bits, some row of x), never memory
  *             outside x; on the other paths such an entry is undefined.  Without row_map it only has
  *             to cover the rows the call reads
@@ -156,10 +156,12 @@ int moe_dispatch_static(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k
  *             scratch; NULL / 0 is accepted (moe_grouped_workspace_bytes reports the reserve)
  *   phases    MOE_PHASE_GATE_UP (writes act), MOE_PHASE_DOWN (reads act, writes y) or
  *             MOE_PHASE_BOTH; the two launches can be issued (and timed) separately
- * Requires h % 64 == 0 and I % 64 == 0, 1 <= E <= 1024.  Which kernel runs follows from n_rows / E alone (from
- * 192 rows per expert, K a multiple of 128 and up to 512 experts: 256-row tiles on persistent workgroups; else one
- * workgroup per tile of 64, 128 or 192 rows, chosen per expert on the device); the two walk k from different stages,
- * so a row's last bit may differ between them, never within one.
+ * Requires h % 64 == 0 and I % 64 == 0, 1 <= E <= 1024.  Two kernels share a call: experts that fit one tile of
+ * 64, 128 or (bf16 weights) 192 rows run one workgroup per tile, at a tile height chosen per expert on the device;
+ * larger experts run on 256-row tiles of persistent workgroups.  From a mean of 1536 rows per expert (n_rows / E) the
+ * persistent kernel takes every expert; below a mean of 128, with K not a multiple of 128, with more than 512
+ * experts or with 4 GiB or more of gathered x, the other one does (larger experts cut into 128-row tiles).  The two
+ * walk k from different stages, so a row's last bit may differ between them, never within one.
  */
 enum { MOE_PHASE_GATE_UP = 1, MOE_PHASE_DOWN = 2, MOE_PHASE_BOTH = 3 };
 size_t moe_grouped_workspace_bytes(int32_t n_rows, int32_t n_experts);

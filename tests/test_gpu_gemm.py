@@ -107,13 +107,13 @@ def test_grouped_odd_stage_counts(E, h, I, counts):
 
 @pytest.mark.parametrize("fp8", [False, True])
 def test_tile_height_follows_the_expert(fp8):
-    """One launch of the one-workgroup-per-tile kernel (mean rows per expert below 192) with experts on both
+    """One launch of the one-workgroup-per-tile kernel alone (mean rows per expert below 128) with experts on both
     sides of every tile-height boundary: a 64-row tile up to 64 rows, one 128-row tile up to 128, one 192-row
     tile up to 192 (bf16 weights only), several 128-row tiles above (those read their weights with plain loads).
     Against the oracle, and an expert's rows bit-for-bit against a launch that holds this expert alone."""
     from moe_gen_amd import ops
-    E, h, I = 12, 512, 384
-    counts = [3, 64, 65, 128, 129, 300, 0, 17, 257, 1, 192, 193]
+    E, h, I = 16, 512, 384
+    counts = [3, 64, 65, 128, 129, 300, 0, 17, 257, 1, 192, 193, 1, 2, 0, 5]
     print(f"tile heights fp8={fp8} counts={counts}", flush=True)
     y, ref32, refr = run_case(E, h, I, counts, fp8, seed=61, use_row_map=True)
     assert np.isfinite(y).all() and rel_max(y, ref32) <= TOL and rel_max(y, refr) <= TOL
@@ -123,9 +123,7 @@ def test_tile_height_follows_the_expert(fp8):
     g = torch.Generator().manual_seed(61)
     x = torch.randn(int(offsets[-1]), h, generator=g).to(torch.bfloat16)
     dev = lambda m: tuple(t.cuda() for t in m) if isinstance(m, tuple) else m.cuda()
-    for e in (1, 2, 4, 10):                              # 64, 65, 129 and 192 rows (alone, 192 rows go to the persistent
-        if counts[e] >= 192:                             # kernel, which walks k in another order)
-            continue
+    for e in (1, 2):                                     # 64 and 65 rows: alone they are below a mean of 128 too
         one = [dev(m) for m in mats[e]]
         if fp8:
             ptrs = ops.expert_pointers([one[0][0]], [one[1][0]], [one[2][0]], [one[0][1]], [one[1][1]], [one[2][1]])
@@ -135,6 +133,38 @@ def test_tile_height_follows_the_expert(fp8):
         ye = ops.grouped_swiglu(x[a:b].cuda(), None, ptrs, torch.tensor([0, b - a], dtype=torch.int32, device="cuda"), b - a)
         torch.cuda.synchronize()
         assert np.array_equal(O.bf16_to_f32(bits(ye)), y[a:b]), f"expert {e} differs from its launch alone"
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_experts_split_between_the_two_kernels(fp8):
+    """Between a mean of 128 and 1536 rows per expert a call launches both kernels and every expert goes by its own
+    count: up to 192 rows (128 with fp8 weights) one tile of the one-workgroup-per-tile kernel, more the persistent
+    kernel's 256-row tiles.  Against the oracle, and every expert's rows bit-for-bit against a call that holds this
+    expert alone (its kernel follows from its count there too, also where the lone call takes another branch of the
+    launcher: 3 rows alone are below a mean of 128, 2000 alone above 1536)."""
+    from moe_gen_amd import ops
+    E, h, I = 9, 256, 384
+    counts = [700, 3, 192, 193, 64, 0, 129, 2000, 128]
+    print(f"two kernels fp8={fp8} counts={counts}", flush=True)
+    y, ref32, refr = run_case(E, h, I, counts, fp8, seed=71, use_row_map=True)
+    assert np.isfinite(y).all() and rel_max(y, ref32) <= TOL and rel_max(y, refr) <= TOL
+    offsets = np.concatenate([[0], np.cumsum(counts)])
+    mats = make_experts(E, h, I, fp8, 72)
+    g = torch.Generator().manual_seed(71)
+    x = torch.randn(int(offsets[-1]), h, generator=g).to(torch.bfloat16)
+    dev = lambda m: tuple(t.cuda() for t in m) if isinstance(m, tuple) else m.cuda()
+    for e in range(E):
+        a, b = int(offsets[e]), int(offsets[e + 1])
+        if b == a:
+            continue
+        one = [dev(m) for m in mats[e]]
+        if fp8:
+            ptrs = ops.expert_pointers([one[0][0]], [one[1][0]], [one[2][0]], [one[0][1]], [one[1][1]], [one[2][1]])
+        else:
+            ptrs = ops.expert_pointers([one[0]], [one[1]], [one[2]])
+        ye = ops.grouped_swiglu(x[a:b].cuda(), None, ptrs, torch.tensor([0, b - a], dtype=torch.int32, device="cuda"), b - a)
+        torch.cuda.synchronize()
+        assert np.array_equal(O.bf16_to_f32(bits(ye)), y[a:b]), f"expert {e} ({b - a} rows) differs from its call alone"
 
 
 @pytest.mark.parametrize("fp8", [False, True])
@@ -278,7 +308,7 @@ def test_expert_sub_range_through_the_persistent_kernel(fp8):
     (512, 128, 128, [200] * 512),             # as many experts as the kernel keeps tables for
 ])
 def test_persistent_kernel_corner_shapes(fp8, E, h, I, counts):
-    """The 256-row persistent kernel (mean rows per expert >= 192, K a multiple of 128) at the ends of what
+    """The 256-row persistent kernel (experts above 192 rows, K a multiple of 128) at the ends of what
     it accepts; rows gathered through a row map."""
     print(f"persistent corners fp8={fp8} E={E} h={h} I={I}", flush=True)
     y, ref32, _ = run_case(E, h, I, counts, fp8, seed=37, use_row_map=True)
