@@ -1046,7 +1046,9 @@ int launch_mt(const GemmArgs& g0, int n_rows, hipStream_t st) {
     // its own height and without 256-row padding, the rest on the persistent kernel's 256-row tiles.  A launch
     // that finds no expert of its kind costs a prefix scan per workgroup.  DeepSeek-V2-Lite, 4096 tokens (64
     // experts of 0 ... 3989 rows, 47 of them below 193, whose 256-row tiles were 49 % padding): block step
-    // 0.923 -> 0.884 ms, routed gate/up 0.388 -> 0.367 ms; DeepSeek-V2-236B, 32768 tokens: 11.48 -> 11.39 ms.
+    // 0.923 -> 0.847 ms, routed gate/up 0.395 -> 0.355 ms; DeepSeek-V2-236B, 32768 tokens: 11.48 -> 11.39 ms.
+    // (The two launches on two streams, so that the second fills the CUs that the persistent kernel's last round
+    // leaves idle, measured the same 0.36 ms: the launches stay on the caller's stream.)
     if (mean >= 1536) {
         g.cold_max = 0;
         return launch_persistent<SWIGLU, W8>(g, n_rows, st);
