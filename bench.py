@@ -230,7 +230,9 @@ def decoder_half_run(w, blk, x, steps: int):
 # (two runs; FETCH_SIZE scaled by 2.0, the factor a plain copy kernel of known size showed on this
 # box, WRITE_SIZE by 1.0).  bench.py cannot run the profiler on itself: these are RECORDED figures,
 # copied from the named summary under profiles/, for the workloads that were profiled; None elsewhere.
-MEASURED_TRAFFIC = {"deepseek_v3_w8a16": (21.3e9, "profiles/pmc_traffic_deepseek_v3_w8a16_65536.md")}
+MEASURED_TRAFFIC = {"deepseek_v3_w8a16": (21.3e9, "profiles/pmc_traffic_deepseek_v3_w8a16_65536.md"),
+                    # 3.03 GiB fetched + the 16 MiB of activations written
+                    "mixtral_8x22b_decode": (3.27e9, "profiles/pmc_small_workloads_decode_and_v2_lite.md")}
 
 
 def run_workload(name: str, args, with_cpu: bool):
@@ -316,7 +318,10 @@ def run_workload(name: str, args, with_cpu: bool):
         roofline = {"bound": "hbm",
                     "kernel": f"grouped_gemm_kernel<WN=4,SWIGLU=true,W8={w8}> (gate/up + SiLU*mul, one workgroup per tile)",
                     "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": gbps / PEAK_HBM_GBPS,
-                    "traffic": None, "launches_per_step": 1, "avg_launch_ms": st["routed_gate_up"],
+                    "traffic": MEASURED_TRAFFIC.get(name, (None, None))[0],
+                    "traffic_source": (f"recorded from {MEASURED_TRAFFIC[name][1]} (rocprofv3 --pmc), not measured by this run"
+                                       if name in MEASURED_TRAFFIC else None),
+                    "launches_per_step": 1, "avg_launch_ms": st["routed_gate_up"],
                     "bytes_per_launch": gu_bytes, "tflops": achieved}
     result = {
         "metric": "MoE-layer tokens/sec at DeepSeek-V3 W8A16 shape" if name == "deepseek_v3_w8a16"
