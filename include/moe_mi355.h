@@ -158,10 +158,13 @@ int moe_dispatch_static(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k
  *             MOE_PHASE_BOTH; the two launches can be issued (and timed) separately
  * Requires h % 64 == 0 and I % 64 == 0, 1 <= E <= 1024.  Two kernels share a call: experts that fit one tile of
  * 64, 128 or (bf16 weights) 192 rows run one workgroup per tile, at a tile height chosen per expert on the device;
- * larger experts run on 256-row tiles of persistent workgroups.  From a mean of 1536 rows per expert (n_rows / E) the
- * persistent kernel takes every expert; below a mean of 128, with K not a multiple of 128, with more than 512
- * experts or with 4 GiB or more of gathered x, the other one does (larger experts cut into 128-row tiles).  The two
- * walk k from different stages, so a row's last bit may differ between them, never within one.
+ * larger experts run on 256-row tiles of persistent workgroups (with fp8 weights: their full 256-row tiles, and the
+ * rows these leave over as one small tile of the first kind if they are at most 128).  With bf16 weights and a mean of
+ * 1536 rows per expert (n_rows / E) or more the persistent kernel takes every expert; below a mean of 128, with K not
+ * a multiple of 128, with more than 512 experts or with 4 GiB or more of gathered x, the other one does (larger
+ * experts cut into 128-row tiles).  An output row's bits depend on the row, its expert's weights and on which of
+ * these branches the call takes, never on the row's place among its expert's rows; between branches the k loop may
+ * start at another stage and a row's last bit may differ.
  */
 enum { MOE_PHASE_GATE_UP = 1, MOE_PHASE_DOWN = 2, MOE_PHASE_BOTH = 3 };
 size_t moe_grouped_workspace_bytes(int32_t n_rows, int32_t n_experts);

@@ -82,6 +82,9 @@ struct GemmArgs {
     int n_tiles_n;              // ceil(N / (SWIGLU ? 128 : 256))
     int cold_max;               // experts of up to this many rows belong to the one-workgroup-per-tile kernel, the
                                 // others to the persistent kernel (0: all to the latter, INT_MAX: all to the former)
+    int rem_split;              // 1: the rule applies to what an expert's full 256-row tiles leave over (count % 256)
+                                // instead of to its count: the persistent kernel takes the full tiles, and the
+                                // last, ragged one only if it holds more than cold_max rows
 };
 
 // LDS rows are 128 bytes = 8 chunks of 16 bytes; chunk c of row r is stored at chunk c ^ swz(r).
@@ -298,9 +301,11 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
     // where it starts, and a column's order depends on nothing but its position, whatever the tile height):
     // Mixtral-8x22B, 256 tokens, down projection 0.302 -> 0.273 ms, gate/up 0.640 -> 0.620 ms.
     // fp8 weights under tiles below 256 rows are fetched 128 k at a time (see PAIR8 below): pairs of stages stay
-    // together, so fp8 tiles start at stage 2 t
+    // together, so fp8 tiles start at stage 2 t.  Not where this kernel takes the rows that the persistent kernel's
+    // full tiles leave over: which of the two computes a row then depends on the row's position among its expert's
+    // rows, so both must add in the same order, the persistent kernel's, from stage 0.
     constexpr bool PAIR8 = W8;
-    const int rot = W8 ? (2 * n_tile) % nk : n_tile % nk;
+    const int rot = g.rem_split ? 0 : W8 ? (2 * n_tile) % nk : n_tile % nk;
     auto stage_at = [&](int kt) { const int kp = kt + rot; return kp >= nk ? kp - nk : kp; };
 
     // ---- per-thread load coordinates ----
@@ -628,7 +633,10 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
 
     // ---- M-tile prefix over experts ----
     ExpertOfThread mine;
-    const int run = mtile_prefix_scan<NT>(g, tid, s_pref, s_wtot, mine, [&](int c) { return c > g.cold_max ? 0 : tiles_of<(W8 ? 128 : 192)>(c); }, [](int, int, int) {});
+    const int run = mtile_prefix_scan<NT>(g, tid, s_pref, s_wtot, mine, [&](int c) {
+        if (g.rem_split) c &= 255;      // the rows the persistent kernel's full tiles leave over
+        return c > g.cold_max ? 0 : tiles_of<(W8 ? 128 : 192)>(c);
+    }, [](int, int, int) {});
     const int total = run * g.n_tiles_n;
 
     // ---- XCD-aware id: groups of 4 consecutive tiles (the M tiles of one N tile first) go round-robin to the XCDs
@@ -664,7 +672,8 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     const int e = uni(s_sel[0]);
     const int pe = uni(s_sel[1]);
     const int mt_e = uni(s_sel[2]);
-    const int first_row = uni(s_sel[3]), row_end = uni(s_sel[4]);
+    const int row_end = uni(s_sel[4]);
+    const int first_row = uni(s_sel[3]) + (g.rem_split ? ((row_end - uni(s_sel[3])) & ~255) : 0);
     int m_tile, n_tile;
     tile_in_expert(v - pe * g.n_tiles_n, mt_e, g.n_tiles_n, m_tile, n_tile);
     if (row_end - first_row <= 64) gemm_tile<1, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
@@ -734,7 +743,10 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
 
     // M-tile prefix over experts; the experts' row offsets and matrix pointers go to LDS tables on the way
     ExpertOfThread mine;
-    const int run = mtile_prefix_scan<NT>(g, tid, s_pref, s_wtot, mine, [&](int c) { return c <= g.cold_max ? 0 : (c + BM - 1) / BM; }, [&](int e, int o0, int o1) {
+    const int run = mtile_prefix_scan<NT>(g, tid, s_pref, s_wtot, mine, [&](int c) {
+        if (g.rem_split) return (c >> 8) + ((c & 255) > g.cold_max ? 1 : 0);
+        return c <= g.cold_max ? 0 : (c + BM - 1) / BM;
+    }, [&](int e, int o0, int o1) {
         s_off[e] = o0;
         if (e == g.E - 1) s_off[g.E] = o1;
         s_ptr[0][e] = (unsigned long long)(uintptr_t)g.b0[e];
@@ -1049,11 +1061,18 @@ int launch_mt(const GemmArgs& g0, int n_rows, hipStream_t st) {
     // 0.923 -> 0.847 ms, routed gate/up 0.395 -> 0.355 ms; DeepSeek-V2-236B, 32768 tokens: 11.48 -> 11.39 ms.
     // (The two launches on two streams, so that the second fills the CUs that the persistent kernel's last round
     // leaves idle, measured the same 0.36 ms: the launches stay on the caller's stream.)
-    if (mean >= 1536) {
+    // fp8 weights: the rule is applied to what an expert's full 256-row tiles leave over, at every mean.  A ragged
+    // last tile costs the persistent kernel a full tile of MFMA time; the other kernel streams the expert's weights
+    // once more for it, and fp8 weights are half the bytes.  DeepSeek-V3, 65536 tokens (256 experts of 581 ... 3941
+    // rows, every second one with at most 128 rows over): block step 46.3 -> 45.8 ms, routed gate/up 25.2 -> 24.8,
+    // down 12.9 -> 12.7 (with up to 64 or 96 rows over 46.2 - 46.3; with all, as two 128-row tiles, 47.1).  With bf16
+    // weights it is break-even (Mixtral-8x7B 9.28 -> 9.23 ms, DeepSeek-V2-236B 11.34 -> 11.42) and not done.
+    if (mean >= 1536 && !W8) {
         g.cold_max = 0;
         return launch_persistent<SWIGLU, W8>(g, n_rows, st);
     }
     g.cold_max = W8 ? 128 : 192;
+    g.rem_split = W8 ? 1 : 0;
     int rc = launch_persistent<SWIGLU, W8>(g, n_rows, st);
     if (rc != MOE_OK) return rc;
     return launch_tiles<4, SWIGLU, W8>(g, n_rows, st);
