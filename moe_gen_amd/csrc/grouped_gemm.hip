@@ -15,13 +15,16 @@
 // expert is cut into M tiles (the last one partial); an M tile times an N tile of the
 // weight matrix is one unit of work.  Every workgroup rebuilds the (tiny) M-tile prefix
 // over experts in LDS from offsets[], so a launch needs neither a host sync nor a tile table.
-// Two kernels:
-//  * grouped_gemm_persistent_kernel (from a mean of 192 rows per expert): 256-row tiles, one
+// Two kernels, and a call usually launches both (launch_mt): every expert goes by its own count, which both
+// kernels read from offsets[]; each builds the prefix over its own share of the tiles.
+//  * grouped_gemm_persistent_kernel (experts above one small tile; with fp8 weights the full 256-row
+//    tiles of every expert): 256-row tiles, one
 //    workgroup per CU, groups of 32 consecutive tiles go round-robin to the XCDs (workgroup
 //    ids are dealt to the 8 XCDs one by one by the hardware; the tiles of a group share their
 //    A and B panels through that XCD's L2), and a workgroup's k pipeline runs on from one of
 //    its tiles into the next.
-//  * grouped_gemm_kernel (fewer rows per expert, a launch that mostly streams weights): one
+//  * grouped_gemm_kernel (experts of up to 192 rows, 128 with fp8 weights, and with fp8 weights what an
+//    expert's full 256-row tiles leave over; work that mostly streams weights): one
 //    workgroup per tile, grid = upper bound on the tile count, surplus workgroups exit at once;
 //    the tile height (64, 128 or 192 rows) follows the expert, groups of 4 tiles go round-robin
 //    to the XCDs.
