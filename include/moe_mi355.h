@@ -162,9 +162,10 @@ int moe_dispatch_static(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k
  * rows these leave over as one small tile of the first kind if they are at most 128).  With bf16 weights and a mean of
  * 1536 rows per expert (n_rows / E) or more the persistent kernel takes every expert; below a mean of 128, with K not
  * a multiple of 128, with more than 512 experts or with 4 GiB or more of gathered x, the other one does (larger
- * experts cut into 128-row tiles).  An output row's bits depend on the row, its expert's weights and on which of
- * these branches the call takes, never on the row's place among its expert's rows; between branches the k loop may
- * start at another stage and a row's last bit may differ.
+ * experts cut into 128-row tiles).  An output row's bits depend on the row and its expert's weights, never on the
+ * row's place among its expert's rows or on any expert's count, with one exception: a call that the
+ * one-workgroup-per-tile kernel serves alone (the last sentence) starts its k loops at other stages, and a row's last
+ * bit may differ from what the other calls give.
  */
 enum { MOE_PHASE_GATE_UP = 1, MOE_PHASE_DOWN = 2, MOE_PHASE_BOTH = 3 };
 size_t moe_grouped_workspace_bytes(int32_t n_rows, int32_t n_experts);

@@ -143,9 +143,9 @@ def test_experts_split_between_the_two_kernels(fp8):
     leave over goes to the other kernel if it is at most 128 rows (300 = 256 + 44, 640 = 512 + 128, 512 leaves
     nothing, 700 = 512 + 188 stays whole).  Against the oracle, and every expert's rows bit-for-bit against a call that
     holds this expert alone (its kernels follow from its count there too, also where the lone call takes another
-    branch of the launcher: 1600 and 2000 rows alone are above a mean of 1536; bf16: 3 rows alone are below a mean of
-    128.  With fp8 weights a lone call below a mean of 128 walks k from another stage than this one, in which both
-    kernels start at stage 0, and is left out)."""
+    branch of the launcher: 1600 and 2000 rows alone are above a mean of 1536.  A lone call below a mean of 128 is
+    served by the one-workgroup-per-tile kernel alone, which then walks k from other stages than a call in which both
+    kernels run and start at stage 0, and is left out)."""
     from moe_gen_amd import ops
     E, h, I = 13, 256, 384
     counts = [700, 3, 192, 193, 64, 0, 129, 2000, 128, 300, 512, 640, 1600]
@@ -159,7 +159,7 @@ def test_experts_split_between_the_two_kernels(fp8):
     dev = lambda m: tuple(t.cuda() for t in m) if isinstance(m, tuple) else m.cuda()
     for e in range(E):
         a, b = int(offsets[e]), int(offsets[e + 1])
-        if b == a or (fp8 and b - a < 128):
+        if b - a < 128:
             continue
         one = [dev(m) for m in mats[e]]
         if fp8:
