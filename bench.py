@@ -292,11 +292,11 @@ def run_workload(name: str, args, with_cpu: bool):
     disp_bytes = w.dispatch_bytes if args.materialize else 4.0 * w.n * w.k
     mean_rows = w.n * w.k // w.E
     # which kernels a grouped GEMM call launches follows from the mean rows per expert (grouped_gemm.hip, launch_mt):
-    # below 128 the one-workgroup-per-tile kernel alone; with bf16 weights from 1536 the persistent kernel alone;
-    # else both (bf16: experts of up to 192 rows on the former; fp8: what an expert's full 256-row tiles leave over,
-    # if at most 128 rows; most rows, and the time, on the latter)
+    # below 128 the one-workgroup-per-tile kernel alone; else both (on the former, bf16: experts of up to 192 rows;
+    # fp8: what an expert's full 256-row tiles leave over, if at most 128 rows; either: the persistent kernel's last
+    # round of tiles if it is at most half a round; most rows, and the time, on the latter)
     persistent = mean_rows >= 128 and w.E <= 512 and w.h % 128 == 0
-    pair = persistent and (w.fp8 or mean_rows < 1536)
+    pair = persistent
     wbytes = 3.0 * w.E * w.h * w.I * (1 if w.fp8 else 2)
     w8 = "true" if w.fp8 else "false"
     if persistent:
@@ -304,7 +304,8 @@ def run_workload(name: str, args, with_cpu: bool):
                     "kernel": f"grouped_gemm_persistent_kernel<SWIGLU=true,W8={w8}> (gate/up + SiLU*mul)"
                               + (f" + grouped_gemm_kernel<WN=4,SWIGLU=true,W8={w8}> for the "
                                  + ("rows past an expert's full 256-row tiles" if w.fp8 else "experts of one small tile")
-                                 + ": a call is this pair of launches, timed as one" if pair else ""),
+                                 + " and a short last round of the persistent kernel: a call is this pair of launches, timed as one"
+                                 if pair else ""),
                     "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": MEASURED_TRAFFIC.get(name, (None, None))[0],
                     "traffic_source": (f"recorded from {MEASURED_TRAFFIC[name][1]} (rocprofv3 --pmc), not measured by this run"

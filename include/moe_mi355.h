@@ -137,11 +137,11 @@ int moe_dispatch_static(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k
  * on bf16 MFMA with fp32 accumulation.
  *   x         device bf16: rows of the sorted token matrix [n_rows, h]; or, when
  *             row_map != NULL, the unsorted matrix, row r being x[row_map[r]]
- *   x_rows    rows of x (>= 1).  It bounds the gather where rows are fetched through a buffer
- *             descriptor (experts on the persistent kernel, below; x smaller than 4 GiB): a row_map entry outside [0, x_rows)
- *             then reads zeros (or, once its byte offset wraps 32 bits, some row of x), never memory
- *             outside x; on the other paths such an entry is undefined.  Without row_map it only has
- *             to cover the rows the call reads
+ *   x_rows    rows of x (>= 1).  It bounds the gather: a row_map entry outside [0, x_rows) stands for a
+ *             row of zeros (where rows are fetched through a buffer descriptor with 32-bit offsets -- the
+ *             persistent kernel, below -- an entry whose byte offset wraps 32 bits reads some row of x
+ *             instead), never memory outside x.  Without row_map it only has to cover the rows the
+ *             call reads
  *   row_map   device int32 [n_rows] or NULL
  *   w_gate/w_up/w_down   device arrays of E device pointers: Wg_e, Wu_e bf16
  *             [I, h]; Wd_e bf16 [h, I]  (nn.Linear [out, in] layout)
@@ -159,13 +159,14 @@ int moe_dispatch_static(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k
  * Requires h % 64 == 0 and I % 64 == 0, 1 <= E <= 1024.  Two kernels share a call: experts that fit one tile of
  * 64, 128 or (bf16 weights) 192 rows run one workgroup per tile, at a tile height chosen per expert on the device;
  * larger experts run on 256-row tiles of persistent workgroups (with fp8 weights: their full 256-row tiles, and the
- * rows these leave over as one small tile of the first kind if they are at most 128).  With bf16 weights and a mean of
- * 1536 rows per expert (n_rows / E) or more the persistent kernel takes every expert; below a mean of 128, with K not
- * a multiple of 128, with more than 512 experts or with 4 GiB or more of gathered x, the other one does (larger
- * experts cut into 128-row tiles).  An output row's bits depend on the row and its expert's weights, never on the
- * row's place among its expert's rows or on any expert's count, with one exception: a call that the
- * one-workgroup-per-tile kernel serves alone (the last sentence) starts its k loops at other stages, and a row's last
- * bit may differ from what the other calls give.
+ * rows these leave over as one small tile of the first kind if they are at most 128).  The persistent workgroups,
+ * one per CU, take whole rounds of tiles; a last round of at most half the CUs' worth of tiles is cut into 128-row
+ * halves and runs with the first kind.  Below a mean of 128 rows per expert (n_rows / E), with K not a multiple of
+ * 128, with more than 512 experts or with 4 GiB or more of gathered x, the one-workgroup-per-tile kernel serves the
+ * call alone (larger experts cut into 128-row tiles).  An output row's bits depend on the row and its expert's
+ * weights, never on the row's place among its expert's rows or on any expert's count, with one exception: a call
+ * that the one-workgroup-per-tile kernel serves alone starts its k loops at other stages, and a row's last bit may
+ * differ from what the other calls give.
  */
 enum { MOE_PHASE_GATE_UP = 1, MOE_PHASE_DOWN = 2, MOE_PHASE_BOTH = 3 };
 size_t moe_grouped_workspace_bytes(int32_t n_rows, int32_t n_experts);

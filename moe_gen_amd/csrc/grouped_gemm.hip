@@ -75,6 +75,7 @@ struct GemmArgs {
     const uint16_t* a;          // activations, row stride K
     const int32_t* row_map;     // optional: sorted row -> row of a
     size_t a_bytes;             // size of a when rows are gathered through row_map
+    int a_rows;                 // rows of a when rows are gathered through row_map
     const void* const* b0;      // per-expert weight matrix [N, K] (gate when SWIGLU, else down)
     const void* const* b1;      // per-expert up matrix [N, K] (SWIGLU only)
     const float* const* s0;     // per-expert block scales of b0 (W8 only)
@@ -88,6 +89,8 @@ struct GemmArgs {
     int rem_split;              // 1: the rule applies to what an expert's full 256-row tiles leave over (count % 256)
                                 // instead of to its count: the persistent kernel takes the full tiles, and the
                                 // last, ragged one only if it holds more than cold_max rows
+    int tail_cus;               // > 0: the persistent kernel runs whole rounds of this many tiles (one per CU); what
+                                // is left, if at most half a round, goes to the other kernel as 128-row half tiles
 };
 
 // LDS rows are 128 bytes = 8 chunks of 16 bytes; chunk c of row r is stored at chunk c ^ swz(r).
@@ -316,10 +319,13 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
     // ---- per-thread load coordinates ----
     const int lrow = tid >> 3, lchunk = tid & 7;          // bf16 tiles: row tid/8 (+RA i), chunk tid%8
     int a_src[NA];
+    bool a_ok[NA];                                        // a row_map entry outside x stands for a row of zeros
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
         int r = min(row0 + lrow + RA * i, row_end - 1);
         a_src[i] = g.row_map ? ((gptr_i32)(uintptr_t)g.row_map)[r] : r;
+        a_ok[i] = !g.row_map || (unsigned)a_src[i] < (unsigned)g.a_rows;
+        if (!a_ok[i]) a_src[i] = 0;
     }
     const uint32_t a_lds = (uint32_t)(lrow * ROW_B + ((lchunk ^ swz(lrow)) << 4));
 
@@ -408,7 +414,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
     auto lds_store = [&](uint8_t* As, int set) {
         uint8_t* Bs = As + A_STAGE;
 #pragma unroll
-        for (int i = 0; i < NA; ++i) *reinterpret_cast<u32x4*>(As + a_lds + i * RA * ROW_B) = ra[set][i];
+        for (int i = 0; i < NA; ++i) *reinterpret_cast<u32x4*>(As + a_lds + i * RA * ROW_B) = a_ok[i] ? ra[set][i] : u32x4{0, 0, 0, 0};
         if (PAIR8) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -523,7 +529,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
         // (PF + 1 stages per tile), so those loads take the first 16 bytes of the activations instead
         const bool past = kt + 1 + PF >= nk;
         if (i < NA) {
-            *reinterpret_cast<u32x4*>(As + a_lds + i * RA * ROW_B) = ra[set][i];
+            *reinterpret_cast<u32x4*>(As + a_lds + i * RA * ROW_B) = a_ok[i] ? ra[set][i] : u32x4{0, 0, 0, 0};
             ra[set][i] = gload16(g.a + (size_t)a_src[i] * K + kofs + lchunk * 8);
         } else if (PAIR8) {
             const int b = i - NA;
@@ -621,6 +627,21 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
 // of 256 CUs and cost 5).  The tiles of an expert that is cut (above 192 rows; above 128 with fp8 weights, where the
 // 192-row body does not fit the registers) run side by side on one XCD and take the weights with plain loads, so
 // that all but the first read of a line come out of that XCD's L2.
+// 256-row tiles of an expert with `count` rows in the persistent kernel's tile space
+__device__ __forceinline__ int persistent_tiles(const GemmArgs& g, int count) {
+    if (g.rem_split) return (count >> 8) + ((count & 255) > g.cold_max ? 1 : 0);
+    return count <= g.cold_max ? 0 : (count + 255) >> 8;
+}
+// How many tiles at the end of that space the persistent kernel leaves to the other kernel.  One workgroup per CU
+// walks the space in rounds of tail_cus tiles, and a last round of a few tiles costs as much as a full one while
+// most CUs idle.  Cut into 128-row halves those tiles occupy twice as many CUs for about 0.7 of a tile's time
+// each, which pays if they are at most half a round.  Both kernels evaluate this on the same offsets[].
+__device__ __forceinline__ int tail_tiles(const GemmArgs& g, int total) {
+    if (g.tail_cus <= 0) return 0;
+    const int tail = total % g.tail_cus;
+    return 2 * tail <= g.tail_cus ? tail : 0;
+}
+
 template <int SINGLE>   // rows that one tile may hold
 __device__ __forceinline__ int tiles_of(int count) { return count <= SINGLE ? (count > 0 ? 1 : 0) : (count + 127) >> 7; }
 
@@ -638,7 +659,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
 
     // ---- M-tile prefix over experts ----
     ExpertOfThread mine;
-    const int run = mtile_prefix_scan<NT>(g, tid, s_pref, s_wtot, mine, [&](int c) {
+    int run = mtile_prefix_scan<NT>(g, tid, s_pref, s_wtot, mine, [&](int c) {
         if (g.rem_split) c &= 255;      // the rows the persistent kernel's full tiles leave over
         return c > g.cold_max ? 0 : tiles_of<(W8 ? 128 : 192)>(c);
     }, [](int, int, int) {});
@@ -649,8 +670,21 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     // weights then share them through one XCD's L2, and dealing small groups round keeps the XCDs even whatever
     // the number of tiles and however much one expert's tiles cost more than another's ----
     const int slot = blockIdx.x >> 3;
-    const int v = (((slot >> 2) << 3) + (blockIdx.x & 7)) * 4 + (slot & 3);
-    if (v >= total) return;
+    int v = (((slot >> 2) << 3) + (blockIdx.x & 7)) * 4 + (slot & 3);
+    // Past this kernel's own tiles: the tiles that the persistent kernel leaves at the end of ITS tile space, two
+    // workgroups (128-row halves, neighbours on one XCD) per tile.  The prefix is rebuilt over that space.
+    int half = -1;
+    if (v >= total) {
+        if (g.tail_cus <= 0 || g.E > NT) return;
+        const int t = v - total;
+        __syncthreads();                 // s_wtot of the first scan has been read by everyone
+        run = mtile_prefix_scan<NT>(g, tid, s_pref, s_wtot, mine, [&](int c) { return persistent_tiles(g, c); }, [](int, int, int) {});
+        const int total_p = run * g.n_tiles_n;
+        const int tail = tail_tiles(g, total_p);
+        if (t >= 2 * tail) return;
+        v = total_p - tail + (t >> 1);
+        half = t & 1;
+    }
     const int q = v / g.n_tiles_n;  // global M-tile number
     // find e with prefix[e] <= q < prefix[e+1].  Up to NT experts every thread still holds its own
     // expert's prefix, tile count and row range: the one that owns q publishes them (one barrier,
@@ -677,10 +711,16 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     const int e = uni(s_sel[0]);
     const int pe = uni(s_sel[1]);
     const int mt_e = uni(s_sel[2]);
-    const int row_end = uni(s_sel[4]);
-    const int first_row = uni(s_sel[3]) + (g.rem_split ? ((row_end - uni(s_sel[3])) & ~255) : 0);
     int m_tile, n_tile;
     tile_in_expert(v - pe * g.n_tiles_n, mt_e, g.n_tiles_n, m_tile, n_tile);
+    if (half >= 0) {                     // half of a 256-row tile of the persistent kernel's space
+        const int r0 = uni(s_sel[3]) + m_tile * 256 + half * 128;
+        const int r1 = min(uni(s_sel[4]), uni(s_sel[3]) + (m_tile + 1) * 256);
+        if (r0 < r1) gemm_tile<2, WN, SWIGLU, W8, false>(g, smem0, smem1, e, r0, r1, n_tile);
+        return;
+    }
+    const int row_end = uni(s_sel[4]);
+    const int first_row = uni(s_sel[3]) + (g.rem_split ? ((row_end - uni(s_sel[3])) & ~255) : 0);
     if (row_end - first_row <= 64) gemm_tile<1, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
     else if (row_end - first_row <= 128) gemm_tile<2, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
     else if (!W8 && mt_e == 1) gemm_tile<3, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
@@ -748,10 +788,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
 
     // M-tile prefix over experts; the experts' row offsets and matrix pointers go to LDS tables on the way
     ExpertOfThread mine;
-    const int run = mtile_prefix_scan<NT>(g, tid, s_pref, s_wtot, mine, [&](int c) {
-        if (g.rem_split) return (c >> 8) + ((c & 255) > g.cold_max ? 1 : 0);
-        return c <= g.cold_max ? 0 : (c + BM - 1) / BM;
-    }, [&](int e, int o0, int o1) {
+    const int run = mtile_prefix_scan<NT>(g, tid, s_pref, s_wtot, mine, [&](int c) { return persistent_tiles(g, c); }, [&](int e, int o0, int o1) {
         s_off[e] = o0;
         if (e == g.E - 1) s_off[g.E] = o1;
         s_ptr[0][e] = (unsigned long long)(uintptr_t)g.b0[e];
@@ -761,7 +798,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
     });
     if (tid == 0) s_pref[g.E] = run;
     __syncthreads();
-    const int total = run * g.n_tiles_n;
+    const int total = run * g.n_tiles_n - tail_tiles(g, run * g.n_tiles_n);   // whole rounds; the rest: the other kernel
     const int xcd = blockIdx.x & 7, slots = gridDim.x >> 3;
     int slot = blockIdx.x >> 3;
     auto tile_of = [&](int sl) { return ((sl / slots) * 8 + xcd) * slots + (sl % slots); };
@@ -1011,7 +1048,8 @@ int launch_tiles(const GemmArgs& g, int n_rows, hipStream_t st) {
     auto kern = grouped_gemm_kernel<WN, SWIGLU, W8>;
     // sum_e tiles_of(c_e) <= sum_e (c_e / 128 + 1); with the larger experts elsewhere, one tile per expert that has rows
     const long max_mtiles = g.cold_max <= 192 ? (g.E < n_rows ? g.E : n_rows) : (long)n_rows / 128 + g.E;
-    const long grid = ((max_mtiles * g.n_tiles_n + 31) / 32) * 32;   // whole rounds of 8 groups of 4 tiles
+    // (+ the persistent kernel's last tiles, at most half a round of them, as two half tiles each)
+    const long grid = ((max_mtiles * g.n_tiles_n + g.tail_cus + 31) / 32) * 32;   // whole rounds of 8 groups of 4 tiles
     if (grid > 0x7fffffffL) {
         set_error("grouped gemm: %ld workgroups exceed the grid limit", grid);
         return MOE_ERR_INVALID;
@@ -1057,27 +1095,29 @@ int launch_mt(const GemmArgs& g0, int n_rows, hipStream_t st) {
         g.cold_max = 0x7fffffff;
         return launch_tiles<4, SWIGLU, W8>(g, n_rows, st);
     }
-    // The counts themselves live on the device; only their mean is known here.  With many rows per expert the
-    // persistent kernel takes them all (an expert's one ragged tile in many).  Else both kernels are launched and
-    // every expert goes by its own count: what fits one tile of the one-workgroup-per-tile kernel runs there, at
-    // its own height and without 256-row padding, the rest on the persistent kernel's 256-row tiles.  A launch
-    // that finds no expert of its kind costs a prefix scan per workgroup.  DeepSeek-V2-Lite, 4096 tokens (64
-    // experts of 0 ... 3989 rows, 47 of them below 193, whose 256-row tiles were 49 % padding): block step
-    // 0.923 -> 0.847 ms, routed gate/up 0.395 -> 0.355 ms; DeepSeek-V2-236B, 32768 tokens: 11.48 -> 11.39 ms.
+    // The counts themselves live on the device; only their mean is known here.  Both kernels are launched and every
+    // expert goes by its own count: what fits one tile of the one-workgroup-per-tile kernel runs there, at its own
+    // height and without 256-row padding, the rest on the persistent kernel's 256-row tiles.  A launch that finds
+    // nothing of its kind costs a prefix scan per workgroup.  DeepSeek-V2-Lite, 4096 tokens (64 experts of
+    // 0 ... 3989 rows, 47 of them below 193, whose 256-row tiles were 49 % padding): block step 0.923 -> 0.847 ms,
+    // routed gate/up 0.395 -> 0.355 ms; DeepSeek-V2-236B, 32768 tokens: 11.48 -> 11.39 ms.
     // (The two launches on two streams, so that the second fills the CUs that the persistent kernel's last round
     // leaves idle, measured the same 0.36 ms: the launches stay on the caller's stream.)
-    // fp8 weights: the rule is applied to what an expert's full 256-row tiles leave over, at every mean.  A ragged
+    // fp8 weights: the rule is applied to what an expert's full 256-row tiles leave over.  A ragged
     // last tile costs the persistent kernel a full tile of MFMA time; the other kernel streams the expert's weights
     // once more for it, and fp8 weights are half the bytes.  DeepSeek-V3, 65536 tokens (256 experts of 581 ... 3941
     // rows, every second one with at most 128 rows over): block step 46.3 -> 45.8 ms, routed gate/up 25.2 -> 24.8,
     // down 12.9 -> 12.7 (with up to 64 or 96 rows over 46.2 - 46.3; with all, as two 128-row tiles, 47.1).  With bf16
     // weights it is break-even (Mixtral-8x7B 9.28 -> 9.23 ms, DeepSeek-V2-236B 11.34 -> 11.42) and not done.
-    if (mean >= 1536 && !W8) {
-        g.cold_max = 0;
-        return launch_persistent<SWIGLU, W8>(g, n_rows, st);
-    }
+    // (Both launches at every mean: from 1536 rows per expert a small expert is rare, but the second launch is there
+    // for the persistent kernel's last round anyway.)
     g.cold_max = W8 ? 128 : 192;
     g.rem_split = W8 ? 1 : 0;
+    // Last round of the persistent kernel (tail_tiles above): Mixtral-8x22B, 8192 tokens, down projection (6.4 rounds
+    // of 0.4 ms) 2.82 -> 2.66 ms, step 8.31 -> 8.13; Mixtral-8x7B 9.39 -> 9.27 ms; DeepSeek-V2-Lite 0.855 -> 0.821 ms
+    // (its shared expert's 128 down tiles become 256 half tiles: 0.071 -> 0.055 ms); DeepSeek-V2-236B 11.43 -> 11.46,
+    // DeepSeek-V3 46.56 -> 46.54: short rounds gain nothing, a partial round of few CUs runs at a higher clock anyway.
+    g.tail_cus = (cu_count() / 8) * 8;     // the persistent launch's grid when there is a round of tiles or more
     int rc = launch_persistent<SWIGLU, W8>(g, n_rows, st);
     if (rc != MOE_OK) return rc;
     return launch_tiles<4, SWIGLU, W8>(g, n_rows, st);
@@ -1104,6 +1144,7 @@ int grouped_swiglu(const void* x, int32_t x_rows, const int32_t* row_map, const 
     g1.a = static_cast<const uint16_t*>(x);
     g1.row_map = row_map;
     g1.a_bytes = (size_t)x_rows * (size_t)hidden * 2;
+    g1.a_rows = x_rows;
     g1.b0 = w_gate; g1.b1 = w_up; g1.s0 = s_gate; g1.s1 = s_up;
     g1.offsets = offsets;
     g1.c = static_cast<uint16_t*>(act);

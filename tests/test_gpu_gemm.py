@@ -172,6 +172,22 @@ def test_experts_split_between_the_two_kernels(fp8):
 
 
 @pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("I,counts", [(1280, [700, 520, 300, 1300, 90]),      # gate/up: 140 tiles, one partial round
+                                      (2560, [700, 520, 300, 1300, 90]),      # gate/up: 280 tiles, a round + 24
+                                      (1664, [2100, 2300, 2500, 1500, 10])])  # gate/up: 442 tiles, a round + 186
+def test_rounds_of_the_persistent_kernel_and_its_last_tiles(fp8, I, counts):
+    """The persistent kernel (one workgroup per CU) takes whole rounds of 256 tiles; a last round of at most 128
+    tiles goes to the other kernel as 128-row halves, a longer one stays (tile counts in the comments: bf16 weights;
+    with fp8 weights, where only an expert's full tiles and ragged tiles above 128 rows count, 110, 220 and 429).  The
+    down projections of these cases have 14 and 34 tiles, all of them half tiles.  Against the oracle."""
+    from moe_gen_amd import ops
+    E, h = len(counts), 256
+    print(f"rounds fp8={fp8} I={I} counts={counts}", flush=True)
+    y, ref32, refr = run_case(E, h, I, counts, fp8, seed=91, use_row_map=True)
+    assert np.isfinite(y).all() and rel_max(y, ref32) <= TOL and rel_max(y, refr) <= TOL
+
+
+@pytest.mark.parametrize("fp8", [False, True])
 @pytest.mark.parametrize("counts", [[300, 640, 129, 70], [2100, 1700], [40, 3, 77]])
 def test_a_row_does_not_depend_on_its_place_in_its_expert(fp8, counts):
     """The same rows in another order within every expert give the same output rows, bit for bit, whichever kernel
@@ -256,16 +272,18 @@ def _one_expert(h, I, seed):
     return ws, ptrs
 
 
-def test_row_map_entry_outside_x_reads_zeros():
-    """The persistent kernel fetches gathered rows through a buffer descriptor that ends with x: a
-    row_map entry beyond x_rows reads a row of zeros (no fault), and every other row is unaffected."""
+@pytest.mark.parametrize("h,I,n", [(256, 256, 600), (256, 8192, 1100), (192, 256, 600), (256, 256, 100)])
+def test_row_map_entry_outside_x_reads_zeros(h, I, n):
+    """A row_map entry beyond x_rows stands for a row of zeros (no fault), and every other row is unaffected: the
+    persistent kernel fetches gathered rows through a buffer descriptor that ends with x (1100 rows x 64 N tiles:
+    a round of its tiles and more), the other kernel checks the entry (600 rows: six tiles, the persistent kernel's
+    short last round as half tiles; K = 192 and 100 rows: calls it serves alone)."""
     from moe_gen_amd import ops
-    h, I, n = 256, 256, 600
     ws, ptrs = _one_expert(h, I, 41)
     g = torch.Generator().manual_seed(42)
     x = torch.randn(n, h, generator=g).to(torch.bfloat16)
     rm = torch.randperm(n, generator=g).to(torch.int32)
-    bad = [3, 257, 599]
+    bad = [3, n // 2 + 7, n - 1]
     rm_bad = rm.clone()
     rm_bad[bad] = torch.tensor([n, n + 5, 2 ** 20], dtype=torch.int32)
     off = torch.tensor([0, n], dtype=torch.int32, device="cuda")
