@@ -138,14 +138,13 @@ def test_tile_height_follows_the_expert(fp8):
 @pytest.mark.parametrize("fp8", [False, True])
 def test_experts_split_between_the_two_kernels(fp8):
     """From a mean of 128 rows per expert a call launches both kernels and every expert goes by its own count.  bf16
-    weights (up to a mean of 1536): up to 192 rows one tile of the one-workgroup-per-tile kernel, more the persistent
-    kernel's 256-row tiles.  fp8 weights: the persistent kernel takes an expert's full 256-row tiles, and what they
-    leave over goes to the other kernel if it is at most 128 rows (300 = 256 + 44, 640 = 512 + 128, 512 leaves
-    nothing, 700 = 512 + 188 stays whole).  Against the oracle, and every expert's rows bit-for-bit against a call that
-    holds this expert alone (its kernels follow from its count there too, also where the lone call takes another
-    branch of the launcher: 1600 and 2000 rows alone are above a mean of 1536.  A lone call below a mean of 128 is
-    served by the one-workgroup-per-tile kernel alone, which then walks k from other stages than a call in which both
-    kernels run and start at stage 0, and is left out)."""
+    weights: up to 192 rows one tile of the one-workgroup-per-tile kernel, more the persistent kernel's 256-row tiles.
+    fp8 weights: the persistent kernel's tile space holds an expert's full 256-row tiles, and what they leave over goes
+    to the other kernel if it is at most 128 rows (300 = 256 + 44, 640 = 512 + 128, 512 leaves nothing, 700 = 512 + 188
+    stays whole).  (At this size the tile space is a short last round, which the other kernel runs as half tiles.)
+    Against the oracle, and every expert's rows bit-for-bit against a call that holds this expert alone, whichever
+    kernel and tile its rows fall to there.  (A lone call below a mean of 128 is served by the one-workgroup-per-tile
+    kernel alone, which then walks k from other stages than a call of both kernels, and is left out.)"""
     from moe_gen_amd import ops
     E, h, I = 13, 256, 384
     counts = [700, 3, 192, 193, 64, 0, 129, 2000, 128, 300, 512, 640, 1600]
