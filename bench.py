@@ -226,6 +226,53 @@ def decoder_half_run(w, blk, x, steps: int):
     return out
 
 
+def calibrate(w, reps: int = 40):
+    """Same-process, same-box yardsticks for the MFMA-bound launches of workload `w`: the vendor library's dense
+    bf16 GEMM (torch.matmul) and this library's own grouped kernel on ONE dense group, both on the workload's
+    gate/up shape ([rows, h] x [2I, h]^T) and down shape ([rows, I] x [h, I]^T) with rows = min(n k, 65536),
+    random operands of the workload's distributions (the chip is power-limited under MFMA load, so operand
+    values matter).  Boxes differ by several per cent in sustained clock; ratios against these figures carry over
+    from box to box, absolute TFLOP/s do not."""
+    import torch
+    from moe_gen_amd import ops
+
+    dev = "cuda:0"
+    rows, h, inter = min(w.n * w.k, 65536), w.h, w.I
+    g = torch.Generator(device=dev).manual_seed(1234)
+    rnd = lambda shape, sd: (torch.randn(shape, generator=g, device=dev) * sd).to(torch.bfloat16)
+    x, w_gu, w_d, act = rnd((rows, h), 1.0), rnd((2 * inter, h), 0.02), rnd((h, inter), 0.02), rnd((rows, inter), 0.05)
+    c1 = torch.empty((rows, 2 * inter), dtype=torch.bfloat16, device=dev)
+    c2 = torch.empty((rows, h), dtype=torch.bfloat16, device=dev)
+    a2 = torch.empty((rows, inter), dtype=torch.bfloat16, device=dev)
+    ptrs = ops.expert_pointers([w_gu[:inter]], [w_gu[inter:]], [w_d])
+    off = torch.tensor([0, rows], dtype=torch.int32, device=dev)
+
+    def timed(fn):
+        # long enough (40 launches after 5 of warm-up, ~0.1 s) for the clock to settle under the load, as it
+        # has in the timed passes of the block
+        for _ in range(5):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / reps
+
+    f_gu, f_d = 4.0 * rows * inter * h, 2.0 * rows * h * inter
+    out = {"vendor_dense_tflops": f_gu / timed(lambda: torch.matmul(x, w_gu.t(), out=c1)) / 1e9,
+           "own_dense_bf16_tflops": f_gu / timed(lambda: ops.grouped_swiglu(x, None, ptrs, off, rows, a2, c2, ops.PHASE_GATE_UP)) / 1e9}
+    a2.copy_(act)
+    out["vendor_dense_down_tflops"] = f_d / timed(lambda: torch.matmul(act, w_d.t(), out=c2)) / 1e9
+    out["own_dense_bf16_down_tflops"] = f_d / timed(lambda: ops.grouped_swiglu(x, None, ptrs, off, rows, a2, c2, ops.PHASE_DOWN)) / 1e9
+    out["shape"] = {"rows": rows, "gate_up": [rows, 2 * inter, h], "down": [rows, h, inter]}
+    out["reps"] = reps
+    del x, w_gu, w_d, act, c1, c2, a2
+    torch.cuda.empty_cache()
+    return out
+
+
 # HBM traffic per launch of the dominant kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (two runs; FETCH_SIZE scaled by 2.0, the factor a plain copy kernel of known size showed on this
 # box, WRITE_SIZE by 1.0).  bench.py cannot run the profiler on itself: these are RECORDED figures,
@@ -251,6 +298,14 @@ def run_workload(name: str, args, with_cpu: bool):
     for _ in range(args.warmup):
         blk(x)
     torch.cuda.synchronize()
+    mean_rows = w.n * w.k // w.E
+    # which kernels a grouped GEMM call launches follows from the mean rows per expert (grouped_gemm.hip, launch_mt):
+    # below 128 the one-workgroup-per-tile kernel alone; else both (on the former, bf16: experts of up to 192 rows;
+    # fp8: what an expert's full 256-row tiles leave over, if at most 128 rows; either: the persistent kernel's last
+    # round of tiles if it is at most half a round; most rows, and the time, on the latter)
+    persistent = mean_rows >= 128 and w.E <= 512 and w.h % 128 == 0
+    # yardsticks of this box, taken right before and right after the timed passes (MFMA-bound workloads)
+    cal = [calibrate(w)] if persistent and not args.no_calibration else []
 
     # the timed region: exactly `steps` passes, nothing but the block's own launches on the stream
     torch.cuda.synchronize()
@@ -274,6 +329,8 @@ def run_workload(name: str, args, with_cpu: bool):
     torch.cuda.synchronize()
     ms_per_step_with_events = (time.perf_counter() - t0) * 1e3 / args.steps
     blk.stage_timer = None
+    if cal:
+        cal.append(calibrate(w))
 
     st = {k: sum(v) / len(v) for k, v in timer.totals_ms().items()}
     # dominant kernel: the fused gate/up SwiGLU GEMM.  With shared experts it is launched twice per
@@ -290,12 +347,6 @@ def run_workload(name: str, args, with_cpu: bool):
     gemm_ms = sum(st.get(k, 0.0) for k in ("routed_gate_up", "routed_down", "shared_gate_up", "shared_down"))
     gemm_tflops = (w.routed_flop + w.shared_flop) / (gemm_ms * 1e-3) / 1e12
     disp_bytes = w.dispatch_bytes if args.materialize else 4.0 * w.n * w.k
-    mean_rows = w.n * w.k // w.E
-    # which kernels a grouped GEMM call launches follows from the mean rows per expert (grouped_gemm.hip, launch_mt):
-    # below 128 the one-workgroup-per-tile kernel alone; else both (on the former, bf16: experts of up to 192 rows;
-    # fp8: what an expert's full 256-row tiles leave over, if at most 128 rows; either: the persistent kernel's last
-    # round of tiles if it is at most half a round; most rows, and the time, on the latter)
-    persistent = mean_rows >= 128 and w.E <= 512 and w.h % 128 == 0
     pair = persistent
     wbytes = 3.0 * w.E * w.h * w.I * (1 if w.fp8 else 2)
     w8 = "true" if w.fp8 else "false"
@@ -313,6 +364,22 @@ def run_workload(name: str, args, with_cpu: bool):
                     "frac_of_fp8_peak": achieved / PEAK_FP8_TFLOPS,
                     "launches_per_step": len(gu_ms), "avg_launch_ms": ms_per_launch,
                     "flop_per_launch": flop_per_launch}
+        if cal:
+            keys = ("vendor_dense_tflops", "own_dense_bf16_tflops", "vendor_dense_down_tflops", "own_dense_bf16_down_tflops")
+            mean = {k: sum(c[k] for c in cal) / len(cal) for k in keys}
+            routed_gu = 4.0 * w.n * w.k * w.h * w.I / (st["routed_gate_up"] * 1e-3) / 1e12
+            routed_dn = 2.0 * w.n * w.k * w.h * w.I / (st["routed_down"] * 1e-3) / 1e12
+            roofline["calibration"] = {**mean, "before_timed_passes": {k: cal[0][k] for k in keys},
+                                       "after_timed_passes": {k: cal[1][k] for k in keys}, "shape": cal[0]["shape"],
+                                       "reps": cal[0]["reps"],
+                                       "what": "same process, same box: vendor library dense bf16 GEMM (torch.matmul) and this "
+                                               "library's grouped kernel on one dense bf16 group, gate/up and down shapes of "
+                                               "this workload, random operands; means of the runs before and after the timed passes"}
+            # the dominant call (all its launches, routed and shared) against the vendor's dense GEMM of the same shape
+            roofline["frac_of_vendor_dense"] = achieved / mean["vendor_dense_tflops"]
+            roofline["own_dense_bf16_frac_of_vendor_dense"] = mean["own_dense_bf16_tflops"] / mean["vendor_dense_tflops"]
+            roofline["routed_gate_up"] = {"tflops": routed_gu, "frac_of_vendor_dense": routed_gu / mean["vendor_dense_tflops"]}
+            roofline["routed_down"] = {"tflops": routed_dn, "frac_of_vendor_dense": routed_dn / mean["vendor_dense_down_tflops"]}
     else:
         # few rows per expert: the launch streams every expert's gate and up matrix once and is bound by HBM.
         # Algorithmic bytes per launch: both matrices of every expert, the gathered token rows, the activations out.
@@ -372,7 +439,7 @@ def ceiling_run(args):
 
     probe = os.path.join(ROOT, "moe_gen_amd", "csrc", "build", "mfma_rate")
     if not os.path.exists(probe):
-        sys.exit(f"{probe} is missing: build it with make -C moe_gen_amd/csrc")
+        sys.exit(f"{probe} is missing: build it with `make -C moe_gen_amd/csrc probes`")
     res = {"metric": "bf16 MFMA ceiling probes (DeepSeek-V3 MoE shapes)", "unit": "TFLOP/s", "peak": PEAK_BF16_TFLOPS}
     # (1) started as a child before this process touches the GPU
     txt = subprocess.run([probe, "10000"], check=True, capture_output=True, text=True, timeout=300).stdout
@@ -462,6 +529,7 @@ def main():
     ap.add_argument("--materialize", action="store_true", help="gather rows into a sorted copy instead of "
                     "reading them through the row map inside the GEMM")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-calibration", action="store_true", help="skip the vendor-dense / own-dense GEMM yardsticks")
     ap.add_argument("--staged", action="store_true", help="also time the block with weights staged from pinned host memory")
     ap.add_argument("--staged-pool", type=int, default=0, help="routed-expert slots of the staging pool (default 20, the reference engine's prefill default)")
     ap.add_argument("--decoder-half", action="store_true", help="also time RMSNorm + block + residual add, fused and separate")

@@ -99,7 +99,8 @@ int moe_router(const void* x, const void* w_gate, const float* bias,
  *   x         device bf16 [n, h]         may be NULL together with xs
  *   xs        device bf16 [n*k, h]  out  gathered rows, may be NULL
  *   workspace device, at least moe_dispatch_workspace_bytes(n, k, E) bytes
- * An id outside [0, E) is not counted and owns no sorted row; its pos entry is 0.
+ * An id outside [0, E) is not counted and owns no sorted row; its pos entry is -1, which
+ * moe_combine skips (the reference would raise an index error on such an id).
  * Limits: 1 <= E <= 256 (the histogram of a block lives in LDS), n * k < 2^31; MOE_ERR_INVALID otherwise.
  */
 size_t moe_dispatch_workspace_bytes(int32_t n_tokens, int32_t top_k, int32_t n_experts);
@@ -119,6 +120,8 @@ int moe_dispatch(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k, int32
  * 65 536 tokens); larger calls fail with MOE_ERR_WORKSPACE and belong to moe_dispatch.  Same
  * kernels, same results as moe_dispatch.  All calls on one GPU share the array: calls that
  * overlap on one GPU (two streams, two threads) race; calls on one stream do not.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress): make that
+ * call eagerly, once per device, before capturing a graph that contains further calls.
  */
 #define MOE_DISPATCH_STATIC_SCRATCH_BYTES (1u << 20)
 int moe_dispatch_static(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k, int32_t n_experts,
@@ -216,7 +219,7 @@ enum {
  * the k slots) and the shared-expert add (modeling_deepseek_v3.py:624-625):
  *     out[t] = sum_j w[t,j] * y[pos[t*k+j]]   (+ shared[t])
  *   y        device bf16 [n*k, h]   expert outputs in sorted-row order
- *   pos      device int32 [n*k]
+ *   pos      device int32 [n*k]     a negative entry contributes nothing (no row of y is read for it)
  *   topk_idx device int32 [n, k]    (needed by MOE_COMBINE_BF16_SEQ only; else may be NULL)
  *   topk_w   device fp32 [n, k]
  *   shared   device bf16 [n, h] or NULL

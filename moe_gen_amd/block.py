@@ -191,7 +191,7 @@ def pool_size(expert, module_type: str = "routed_expert") -> int:
     return 1
 
 
-def expert_waves(n_experts: int, pool: int, hot=None):
+def expert_waves(n_experts: int, pool: int, hot=None, backed=None):
     """Cut a layer's experts into waves for a pool of `pool` slots.
 
     Returns a list of (first, last_plus_one, fetch_list): the grouped kernels of a wave run on the
@@ -204,11 +204,24 @@ def expert_waves(n_experts: int, pool: int, hot=None):
     Without `hot` every expert is fetched, in id order -- the order in which the copy worker delivers
     them, so a wave's weights are exactly what the pool holds or receives next.  With `hot` (ids of the
     experts that received tokens, on-demand staging) only those are fetched; a wave then spans from its
-    first to its last hot expert and the cold ones in between own no rows."""
+    first to its last hot expert and the cold ones in between own no rows.
+    `backed` (ids of the experts whose weights come from the engine; the others are resident, the
+    reference decides expert by expert, deepseekv3_initializer.py:1259-1266) restricts the fetch lists
+    to those ids, and the waves then cover every expert: the first starts at expert 0, each ends where
+    the next one starts and the last at n_experts, so that resident experts run in the wave they fall into."""
     pool = max(1, int(pool))
     ids = list(range(n_experts)) if hot is None else sorted(hot)
+    if backed is not None:
+        keep = set(backed)
+        ids = [e for e in ids if e in keep]
     step = pool if len(ids) <= pool else max(1, pool // 2)
-    return [(ids[i], ids[min(i + step, len(ids)) - 1] + 1, ids[i:i + step]) for i in range(0, len(ids), step)]
+    waves = [(ids[i], ids[min(i + step, len(ids)) - 1] + 1, ids[i:i + step]) for i in range(0, len(ids), step)]
+    if backed is None:
+        return waves
+    if not waves:
+        return [(0, n_experts, [])]
+    starts = [0] + [w[0] for w in waves[1:]] + [n_experts]
+    return [(starts[i], starts[i + 1], w[2]) for i, w in enumerate(waves)]
 
 
 def staged_experts_forward(experts, launch, counts_host=None, on_demand=False, stream_wait=None, module_type="routed_expert"):
@@ -222,13 +235,21 @@ def staged_experts_forward(experts, launch, counts_host=None, on_demand=False, s
     host and its copy thread overwrites it immediately (GPU_Weight_Buffer.cpp:163-169), which is
     why Expert_Wrapper synchronises before free_weights_buffer (Wrapper.py:512-517).
 
+    Experts are taken one by one (the reference wraps every expert and sets `get_weights` per expert,
+    Mixtral_Initializer.py:761-787, deepseekv3_initializer.py:1259-1266): one with `get_weights`
+    false keeps its weights resident and runs in the wave its id falls into.
+
     counts_host: per-expert token counts on the host; needed when there is more than one wave (the
     launch of a wave is sized by its own rows) and for on-demand staging.
     on_demand: fetch only experts with tokens through the engine's `fetch` (busiest first when
     they fit the pool at once)."""
-    first = experts[0]
-    eng = first.core_engine
     E = len(experts)
+    backed = [e for e in range(E) if engine_backed(experts[e])]
+    if not backed:
+        raise RuntimeError("staged_experts_forward: no expert of the layer takes its weights from an engine")
+    mixed = len(backed) < E
+    first = experts[backed[0]]
+    eng = first.core_engine
     pool = pool_size(first, module_type)
     routed = getattr(first, "expert_idx", -1) != -1
     if routed:
@@ -237,28 +258,38 @@ def staged_experts_forward(experts, launch, counts_host=None, on_demand=False, s
         eng.clear_expert_buffer(first.layer_idx, 0)
     hot = None
     if on_demand and counts_host is not None and hasattr(eng, "fetch"):
-        hot = [e for e in range(E) if counts_host[e] > 0]
-        if not hot:
+        hot = [e for e in backed if counts_host[e] > 0]
+        if not hot and not mixed:
             return
-        if len(hot) <= pool:
+        if hot and len(hot) <= pool:
             hot_by_load = sorted(hot, key=lambda e: -counts_host[e])
             eng.fetch([experts[e].expert_weights_idx for e in hot_by_load])
-    waves = expert_waves(E, pool, hot)
+    waves = expert_waves(E, pool, hot, backed if mixed else None)
     if len(waves) > 1 and counts_host is None:
         raise RuntimeError("staged_experts_forward: more than one wave needs the per-expert counts on the host")
     ordered = bool(getattr(eng, "stream_ordered_release", False))
     on_demand_waves = hot is not None and len(hot) > pool
-    if on_demand_waves:                                      # the first wave's copies; each wave then asks for the next one's
+    # a wave is half the pool, so the next wave's copies go into the half this wave does not hold; a pool of a
+    # single slot has no other half, and its next copy can only be asked for once the slot has been let go
+    ahead = on_demand_waves and all(len(a[2]) + len(b[2]) <= pool for a, b in zip(waves, waves[1:]))
+    if on_demand_waves and ahead:                            # the first wave's copies; each wave then asks for the next one's
         eng.fetch([experts[e].expert_weights_idx for e in waves[0][2]])
+    resident_rows = {e: _tensors_of(experts[e]) for e in range(E) if e not in set(backed)} if mixed else {}
     for w, (a, b, fetch) in enumerate(waves):
-        if on_demand_waves and w + 1 < len(waves):           # into the half of the pool this wave does not hold
-            eng.fetch([experts[e].expert_weights_idx for e in waves[w + 1][2]])
+        if on_demand_waves:
+            if not ahead:
+                eng.fetch([experts[e].expert_weights_idx for e in fetch])
+            elif w + 1 < len(waves):
+                eng.fetch([experts[e].expert_weights_idx for e in waves[w + 1][2]])
         got = {e: _tensors_of(experts[e], eng.get_weights(experts[e].expert_weights_idx)) for e in fetch}
-        stand_in = got[fetch[0]]                             # an expert without rows is never read
+        got.update({e: resident_rows[e] for e in range(a, b) if e in resident_rows})
+        if not got:                                          # nothing but engine-backed experts without rows
+            continue
+        stand_in = next(iter(got.values()))                  # an expert without rows is never read
         rows = [got.get(e, stand_in) for e in range(a, b)]
         n_rows = None if counts_host is None else int(sum(counts_host[a:b]))
         launch(rows, a, b, n_rows)
-        if not ordered and stream_wait is not None:
+        if not ordered and stream_wait is not None and fetch:
             stream_wait()
         for e in fetch:
             eng.free_weights_buffer(experts[e].expert_weights_idx)
@@ -281,13 +312,14 @@ def _gate_weight_bf16(weight: torch.Tensor, cache: dict) -> torch.Tensor:
 
 def _engine_experts(block, timer, tag, experts, a_rows, row_map, offsets, n_rows, counts):
     """The expert MLPs of one layer with weights handed out by an engine, wave by wave."""
-    first = experts[0]
+    first = next(ex for ex in experts if engine_backed(ex))
     routed = tag == "routed"
     mtype = "routed_expert" if routed else "shared_expert"
     E = len(experts)
     aware = routed and bool(getattr(block, "routing_aware_staging", False)) and hasattr(first.core_engine, "fetch")
     counts_host = None
-    if routed and (aware or pool_size(first, mtype) < E):
+    n_backed = sum(1 for ex in experts if engine_backed(ex))
+    if routed and (aware or pool_size(first, mtype) < n_backed):
         counts_host = counts.tolist()                        # one read of E integers (the reference reads them too, :673)
     hidden, inter = a_rows.shape[1], None
     act = y = None
@@ -351,7 +383,7 @@ def moe_forward(block, hidden_states: torch.Tensor, spec: ops.RouterSpec, gate_w
     block.last_counts = counts
     experts = list(experts)
     a_rows = x if fused_gather else d.xs
-    if engine_backed(experts[0]):
+    if any(engine_backed(ex) for ex in experts):   # decided expert by expert, as the reference's initializers do
         y = _engine_experts(block, timer, "routed", experts, a_rows, row_map, offsets, n * k, counts)
     else:
         y = _grouped(timer, "routed", a_rows, row_map, collect_pointers(experts, cache.setdefault("routed", {})),

@@ -57,10 +57,16 @@ __global__ __launch_bounds__(1024) void combine_kernel(const u32x4* __restrict__
         for (int a0 = 0; a0 < k; a0 += KB) {
         u32x4 vb[KB];
 #pragma unroll
-        for (int b = 0; b < KB; ++b) vb[b] = __builtin_nontemporal_load(&y[(size_t)s_row[min(a0 + b, k - 1)] * chunks + c]);   // past k: the last row again
+        for (int b = 0; b < KB; ++b) {
+            // past k: the last row again; a negative row (a slot whose expert id moe_dispatch found outside
+            // [0, E)) is neither read nor added -- the same for every lane of the block
+            const int row = s_row[min(a0 + b, k - 1)];
+            vb[b] = row < 0 ? u32x4{0, 0, 0, 0} : __builtin_nontemporal_load(&y[(size_t)row * chunks + c]);
+        }
 #pragma unroll
         for (int b = 0; b < KB; ++b) {
             if (a0 + b >= k) break;
+            if (s_row[a0 + b] < 0) continue;
             const u32x4 v = vb[b];
             const float w = s_w[a0 + b];
 #pragma unroll

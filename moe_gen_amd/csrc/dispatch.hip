@@ -133,9 +133,9 @@ __global__ __launch_bounds__(256) void rank_scatter(const int32_t* __restrict__ 
         const bool in_list = g < nk;
         int e = in_list ? idx[g] : 0;
         const bool ok = in_list && (unsigned)e < (unsigned)E;
-        // an expert id outside [0, E) owns no sorted row: its slot points at row 0 so that a
-        // combine over this list reads valid memory
-        if (in_list && !ok) pos[g] = 0;
+        // an expert id outside [0, E) owns no sorted row: its slot gets -1, which the combine
+        // skips (no row read, nothing added)
+        if (in_list && !ok) pos[g] = -1;
         uint64_t peers = __ballot(ok);
 #pragma unroll
         for (int b = 0; b < 8; ++b) {

@@ -42,6 +42,7 @@ struct Module {
     std::vector<Piece> pieces;
     int slot = -1;               // -1: not resident
     bool held = false;           // acquired by a consumer and not yet released
+    bool wanted = false;         // named by a fetch and not yet released (on-demand staging)
     int layer = -1, expert = -2; // tag: routed expert `expert` (>= 0) or shared expert (-1) of `layer`; -2 untagged
     hipEvent_t ready = nullptr;  // copy finished (device backend)
 };
@@ -133,16 +134,34 @@ int pump_type(moe_stager* st, int ti) {
 // on-demand copy of one module; 1 if enqueued, 0 if already resident, <0 on error
 int fetch_one(moe_stager* st, int id) {
     Module& m = st->modules[id];
-    if (m.slot >= 0) return 0;
+    if (m.slot >= 0) {
+        m.wanted = true;
+        return 0;
+    }
     Type& t = st->types[m.type];
-    const int slot = find_free(t);
+    int slot = find_free(t);
     if (slot < 0) {
-        moe::set_error("moe_stage_fetch: no free slot of type %d for module %d (%d active slots, all held)", m.type, id,
-                       t.n_active);
+        // A slot whose module nobody has acquired and no fetch has named -- left there by the cyclic prefetch before
+        // the type was switched to on-demand, or by an earlier call's surplus -- is taken over: no consumer reads
+        // it, and the new copy follows the old one on the copy stream.
+        for (int s = 0; s < t.n_active && slot < 0; ++s) {
+            Module& o = st->modules[t.owner[s]];
+            if (!o.held && !o.wanted) {
+                o.slot = -1;
+                t.owner[s] = -1;
+                slot = s;
+            }
+        }
+    }
+    if (slot < 0) {
+        moe::set_error("moe_stage_fetch: no free slot of type %d for module %d (%d active slots, all held or named by "
+                       "an earlier fetch)", m.type, id, t.n_active);
         return MOE_ERR_STATE;
     }
     int rc = copy_into(st, id, slot);
-    return rc != MOE_OK ? rc : 1;
+    if (rc != MOE_OK) return rc;
+    m.wanted = true;
+    return 1;
 }
 
 // hand the slot of a resident module back; the next copy into it waits for `stream`
@@ -156,6 +175,7 @@ int release_one(moe_stager* st, int id, hipStream_t stream) {
     t.owner[m.slot] = -1;
     m.slot = -1;
     m.held = false;
+    m.wanted = false;
     return MOE_OK;
 }
 
@@ -170,7 +190,10 @@ int drop_residency(moe_stager* st, int ti, const char* who) {
         }
     if (st->backend == MOE_STAGE_DEVICE) MOE_HIP_CHECK(hipStreamSynchronize(st->copy_stream));
     for (int s = 0; s < t.n_total; ++s) {
-        if (t.owner[s] >= 0) st->modules[t.owner[s]].slot = -1;
+        if (t.owner[s] >= 0) {
+            st->modules[t.owner[s]].slot = -1;
+            st->modules[t.owner[s]].wanted = false;
+        }
         t.owner[s] = -1;
     }
     return MOE_OK;
@@ -332,16 +355,20 @@ extern "C" int moe_stage_clear_expert_buffer(moe_stager* st, int32_t layer_idx, 
     std::lock_guard<std::mutex> lk(st->mu);
     const int prev = (layer_idx >= 0 && layer_idx < st->wrap_layers) ? st->num_hidden_layers - 1 : layer_idx - 1;
     int n = 0;
-    for (size_t id = 0; id < st->modules.size(); ++id) {
-        Module& m = st->modules[id];
-        if (m.slot < 0 || m.expert < 0) continue;                   // not resident / not a routed expert
-        const bool earlier = m.layer == layer_idx && m.expert < expert_idx;
-        const bool previous = m.layer == prev && m.expert < st->num_local_experts;
-        if (!earlier && !previous) continue;
-        int rc = release_one(st, (int)id, moe::as_stream(stream));
-        if (rc != MOE_OK) return rc;
-        ++n;
-    }
+    // only resident modules can be released: walk the slots (a few dozen), not the modules (thousands in a model)
+    for (Type& t : st->types)
+        for (int s = 0; s < t.n_total; ++s) {
+            const int id = t.owner[s];
+            if (id < 0) continue;
+            Module& m = st->modules[id];
+            if (m.expert < 0) continue;                                 // not a routed expert
+            const bool earlier = m.layer == layer_idx && m.expert < expert_idx;
+            const bool previous = m.layer == prev && m.expert < st->num_local_experts;
+            if (!earlier && !previous) continue;
+            int rc = release_one(st, id, moe::as_stream(stream));
+            if (rc != MOE_OK) return rc;
+            ++n;
+        }
     if (n > 0) {
         int r = pump_all(st);
         if (r < 0) return r;

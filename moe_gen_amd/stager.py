@@ -158,8 +158,10 @@ class Stager:
         return mid
 
     def pool_size(self, module_type: str) -> int:
-        """Slots of `module_type` usable in the current phase."""
-        return (self.n_decoding if self.phase == "decoding" else self.n_prefill)[module_type]
+        """Slots of `module_type` usable in the current phase (the rule the pools were sized by: a type
+        without a decoding entry keeps its prefill slots, and the decoding pool never shrinks)."""
+        n = self.n_prefill[module_type]
+        return max(n, self.n_decoding.get(module_type, 0)) if self.phase == "decoding" else n
 
     def set_policy(self, module_type: str, policy: str) -> None:
         """"cyclic": every module of the type is copied in registration order whether or not it

@@ -67,8 +67,8 @@ def test_dispatch_full_size_properties():
 
 
 def test_dispatch_ignores_out_of_range_ids():
-    """Ids outside [0, E) are not counted, own no sorted row and get pos 0, so a combine over the
-    list reads valid memory; the in-range entries are ranked as if the others were absent."""
+    """Ids outside [0, E) are not counted, own no sorted row and get pos -1, which the combine skips;
+    the in-range entries are ranked as if the others were absent."""
     from moe_gen_amd import ops
     E, k = 16, 2
     idx = rand_idx(200, k, E, 5)
@@ -84,7 +84,23 @@ def test_dispatch_ignores_out_of_range_ids():
     order = np.flatnonzero(good)[np.argsort(flat[good], kind="stable")]
     assert np.array_equal(perm.cpu().numpy()[:n_good], order)
     p = pos.cpu().numpy()
-    assert np.array_equal(p[order], np.arange(n_good)) and (p[~good] == 0).all()
+    assert np.array_equal(p[order], np.arange(n_good)) and (p[~good] == -1).all()
+    # through the combine: a skipped slot adds nothing, i.e. the result equals the oracle's on a list in which
+    # those slots point at a row of zeros with weight zero (x + 0 * 0 == x); the rows of y behind no slot hold NaN
+    h = 256
+    g = torch.Generator().manual_seed(3)
+    ys = torch.full((flat.size, h), float("nan")).to(torch.bfloat16)
+    ys[:n_good] = torch.randn(n_good, h, generator=g).to(torch.bfloat16)
+    w = torch.rand(200, k, generator=g) * 2.5
+    ys_ref = torch.cat([ys[:n_good], torch.zeros(1, h, dtype=torch.bfloat16)])
+    pos_ref, w_ref, idx_ref = p.copy(), w.numpy().copy(), bad.copy()
+    pos_ref[~good] = n_good
+    w_ref.reshape(-1)[~good] = 0.0
+    for mode in (0, 1, 2):
+        out = ops.combine(ys.cuda(), pos, torch.from_numpy(bad).cuda(), w.cuda(), None, mode)
+        torch.cuda.synchronize()
+        ref = O.combine(bits(ys_ref), pos_ref, idx_ref, w_ref, None, mode)
+        assert np.array_equal(bits(out), ref), mode
 
 
 @pytest.mark.parametrize("mode", [0, 1, 2])

@@ -213,3 +213,87 @@ def test_on_demand_waves_fetch_only_experts_with_tokens():
     launches.clear()
     block.staged_experts_forward(experts, lambda rows, a, b, n: launches.append((a, b, n)), few, on_demand=True)
     assert launches == [(2, 9, 10)] and not eng.held
+
+
+@pytest.mark.parametrize("slots", [1, 2, 3])
+def test_on_demand_waves_with_a_tiny_pool(slots):
+    """More hot experts than slots: a wave is half the pool and the next wave is asked for while this
+    one is multiplied -- except with a single slot, which has no other half: its next copy is asked
+    for only after the slot has been let go.  Against the stand-in engine and against the library's
+    Stager (host backend), whose fetch fails when no slot is free."""
+    from moe_gen_amd import Stager, block
+    E, L = 7, 3
+    counts = [2, 0, 5, 1, 0, 3, 4]
+    hot = [e for e in range(E) if counts[e]]
+    eng = _SlotLimitedEngine([f"routed_expert_{L}_{e}" for e in range(E)], slots, on_demand=True)
+    eng.pool_size = lambda module_type: slots
+    eng.stream_ordered_release = True
+    launches = []
+    block.staged_experts_forward([_Wrapped(eng, L, e) for e in range(E)], lambda rows, a, b, n: launches.append((a, b, n)),
+                                 counts, on_demand=True)
+    assert sum(n for _, _, n in launches) == sum(counts) and not eng.held and not eng.resident
+    assert [c[1] for c in eng.calls if c[0] == "get"] == [f"routed_expert_{L}_{e}" for e in hot]
+
+    shapes = {"routed_expert": {f"{n}.weight": ((2, 2), torch.float32) for n in _Wrapped.names}}
+    st = Stager(shapes, {"routed_expert": slots}, backend="host", model_type="mixtral", num_hidden_layers=L + 1,
+                num_local_experts=E)
+    st.set_policy("routed_expert", "on_demand")
+    for e in range(E):
+        st.add_module(f"routed_expert_{L}_{e}", "routed_expert",
+                      {f"{n}.weight": torch.full((2, 2), float(e)) for n in _Wrapped.names})
+    seen = []
+
+    def launch(rows, a, b, n):
+        for e in range(a, b):
+            if counts[e]:
+                seen.append((e, float(rows[e - a][0][0, 0])))          # the gate matrix handed out for expert e
+
+    for rep in range(2):
+        seen.clear()
+        block.staged_experts_forward([_Wrapped(st, L, e) for e in range(E)], launch, counts, on_demand=True)
+        assert seen == [(e, float(e)) for e in hot]
+        assert st.stats()[0] == (rep + 1) * len(hot)
+        assert not any(st.resident(f"routed_expert_{L}_{e}") for e in range(E))
+
+
+def test_layer_with_resident_and_engine_backed_experts():
+    """The reference sets get_weights expert by expert (Mixtral_Initializer.py:761-787,
+    deepseekv3_initializer.py:1259-1266): experts outside the copy task keep their weights.  Only the
+    engine-backed ones count against the pool, every expert lands in exactly one wave, and a resident
+    expert is never asked of the engine."""
+    from moe_gen_amd import block
+    E, slots, L = 9, 4, 2
+    backed = [1, 2, 4, 5, 6, 8]
+    eng = _SlotLimitedEngine([f"routed_expert_{L}_{e}" for e in backed], slots)
+    experts = [_Wrapped(eng, L, e, _engine_config(slots, slots)) for e in range(E)]
+    for e in range(E):
+        if e not in backed:
+            experts[e].get_weights = False
+            experts[e].gate_proj.weight.data.fill_(100.0 + e)
+    counts = [3, 1, 0, 2, 5, 1, 1, 4, 2]
+    covered, launches = [], []
+
+    def launch(rows, a, b, n):
+        launches.append((a, b, n))
+        for e in range(a, b):
+            covered.append(e)
+            if e in backed:
+                assert f"routed_expert_{L}_{e}" in eng.held
+            else:
+                assert float(rows[e - a][0][0, 0]) == 100.0 + e       # its own resident gate matrix
+        eng.synced = False
+
+    def stream_wait():
+        eng.synced = True
+
+    block.staged_experts_forward(experts, launch, counts, stream_wait=stream_wait)
+    assert covered == list(range(E)) and sum(n for _, _, n in launches) == sum(counts)
+    assert [c[1] for c in eng.calls if c[0] == "get"] == [f"routed_expert_{L}_{e}" for e in backed]
+    assert not eng.held
+    assert block.expert_waves(9, 4, backed=backed) == [(0, 4, [1, 2]), (4, 6, [4, 5]), (6, 9, [6, 8])]
+    assert block.expert_waves(9, 8, backed=backed) == [(0, 9, backed)]
+    assert block.expert_waves(4, 2, hot=[], backed=[1, 3]) == [(0, 4, [])]
+    with pytest.raises(RuntimeError, match="no expert of the layer"):
+        for ex in experts:
+            ex.get_weights = False
+        block.staged_experts_forward(experts, launch, counts)

@@ -231,3 +231,48 @@ def test_on_demand_fetches_only_what_is_named():
     st.free_weights_buffer("routed_expert_1_7")
     st.set_policy("routed_expert", "cyclic")
     assert st.pump() == slots and st.resident("routed_expert_0_0")
+
+
+def test_fetch_takes_over_slots_nobody_asked_for():
+    """Slots filled by the cyclic prefetch before a type was switched to on-demand hold modules that
+    no consumer acquired and no fetch named: a fetch that finds no free slot takes those over instead
+    of failing, but never a held module or one an earlier fetch named."""
+    E, slots = 6, 3
+    st = Stager(SHAPES, {"routed_expert": slots, "shared_expert": 1}, backend="host", model_type="mixtral",
+                num_hidden_layers=2, num_local_experts=E)
+    host = {}
+    for L in range(2):
+        for e in range(E):
+            key = f"routed_expert_{L}_{e}"
+            host[key] = {n: torch.full(s, float(10 * L + e)).to(d) for n, (s, d) in SHAPES["routed_expert"].items()}
+            st.add_module(key, "routed_expert", host[key])
+    assert st.pump() == slots                               # cyclic: experts 0..2 of layer 0 fill the pool
+    st.set_policy("routed_expert", "on_demand")
+    assert st.fetch(["routed_expert_1_4", "routed_expert_1_5"]) == 2     # two of the three prefetched modules give way
+    assert sum(st.resident(f"routed_expert_0_{e}") for e in range(3)) == 1
+    w = st.get_weights("routed_expert_1_4")
+    assert float(w["gate_proj.weight"][0, 0]) == 14.0
+    assert st.fetch(["routed_expert_1_0"]) == 1             # the last prefetched module gives way
+    assert not any(st.resident(f"routed_expert_0_{e}") for e in range(3))
+    with pytest.raises(RuntimeError, match="no free slot"):  # held (1_4) and named (1_5, 1_0) modules stay
+        st.fetch(["routed_expert_1_1"])
+    st.free_weights_buffer("routed_expert_1_4")
+    assert st.fetch(["routed_expert_1_1"]) == 1
+    for key in ("routed_expert_1_5", "routed_expert_1_0", "routed_expert_1_1"):
+        w = st.get_weights(key)
+        assert all(torch.equal(w[n], host[key][n]) for n in w)
+        st.free_weights_buffer(key)
+
+
+def test_pool_size_in_the_decoding_phase_follows_the_pool():
+    """A type without a decoding entry keeps its prefill slots; a decoding count below the prefill
+    count does not shrink the pool (the C side runs with the larger of the two)."""
+    st = Stager(SHAPES, {"routed_expert": 4, "shared_expert": 2}, n_slots_decoding={"routed_expert": 3}, backend="host",
+                model_type="mixtral", num_hidden_layers=1, num_local_experts=4)
+    st.set_phase("decoding")
+    assert st.pool_size("routed_expert") == 4 and st.pool_size("shared_expert") == 2
+    st2 = Stager(SHAPES, {"routed_expert": 2, "shared_expert": 1}, n_slots_decoding={"routed_expert": 6}, backend="host",
+                 model_type="mixtral", num_hidden_layers=1, num_local_experts=4)
+    assert st2.pool_size("routed_expert") == 2
+    st2.set_phase("decoding")
+    assert st2.pool_size("routed_expert") == 6 and st2.pool_size("shared_expert") == 1
