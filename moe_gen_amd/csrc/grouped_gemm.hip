@@ -105,6 +105,7 @@ __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1
 typedef const __attribute__((address_space(1))) u32x4* gptr_u32x4;
 typedef const __attribute__((address_space(1))) float* gptr_f32;
 typedef const __attribute__((address_space(1))) int32_t* gptr_i32;
+typedef __attribute__((address_space(3))) uint8_t* lds_u8;
 
 __device__ __forceinline__ u32x4 gload16(const void* p) { return *(gptr_u32x4)(uintptr_t)p; }
 // Weights under the one-workgroup-per-tile kernel are streamed: a tile of them is used by one workgroup (two
@@ -620,6 +621,191 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
                                                        min(BM, row_end - row0) - wm * 32 * MT, N - ncol0);
 }
 
+// ---- fp8 weight streamer: experts of up to 64 rows in calls that the one-workgroup-per-tile kernel serves alone ----
+//
+// With a handful of rows per expert a launch reads every weight once (Expert_Wrapper.forward in its decoding use,
+// Wrapper.py:470-530) and is bound by how fast a CU can take fp8 weights in.  Through gemm_tile a 64-k stage of 256
+// weight rows costs 16 KiB of global loads into registers, the conversion, 32 KiB of LDS stores, a barrier and
+// 64 KiB of fragment reads, and streams at 4-5 TB/s.  Here
+//  * the workgroup's 8 waves split the tile's WEIGHT rows (32 each: a 16-row gate fragment and the matching up
+//    fragment, or two fragments of the down matrix) and every wave multiplies all token rows, so a weight is
+//    converted once, by the wave that feeds it to the matrix core;
+//  * weights reach LDS as fp8 by DMA (buffer_load ... lds), 8 lanes x 16 bytes per row = whole 128-byte lines per
+//    request, 128 k at a time, into the wave's own 4 KiB of a buffer: no staging registers, no LDS stores, half the
+//    bytes, and three buffers keep two 128-k blocks in flight per CU;
+//  * a lane reads 16 consecutive fp8 weights of its fragment row (one ds_read_b128), which after conversion are its
+//    A operands of BOTH 32-wide k-steps of a 64-k half: lane group q holds k = 16 q + 8 s + (0..7) in step s, and the
+//    token operand reads the chunk that holds those k.  A dot product does not care in which order k is walked,
+//    and the order depends on nothing but the column: a row's result does not depend on its tile or its neighbours.
+// LDS layouts (the DMA lets every lane fetch what belongs at its place, so swizzles are free):
+//  weights: 128-byte rows, 16-byte part c of fragment row r at part c ^ wsw(r); tokens: 256-byte rows (128 k), chunk
+//  c of row r at chunk c ^ tsw(r).  The LDS serves lanes 8 i .. 8 i + 7 together with lanes 32 + 8 i .. (the same 8
+//  rows, lane groups q and q + 2): with these keys their 16 reads fall on 16 different bank groups.
+__device__ __forceinline__ int wsw(int r) { return ((r >> 1) & 1) | (((r >> 2) & 1) << 2); }
+__device__ __forceinline__ int tsw(int r) { return (r & 3) | ((r & 4) << 1); }
+
+constexpr int S8_WBYTES = 32 * 1024;              // weight region of a buffer: 8 waves x 32 rows x 128 fp8
+constexpr int S8_TROWS = 64;                      // token rows staged
+constexpr int S8_BUF = S8_WBYTES + S8_TROWS * 256;
+
+template <int TG, bool SWIGLU>   // TG: 16-row token groups multiplied (the expert has at most 16 TG <= 64 rows)
+__device__ __forceinline__ void stream8_tile(const GemmArgs& g, uint8_t* buf0, uint8_t* buf1, uint8_t* buf2, int e, int row0,
+                                             int row_end, int n_tile) {
+    constexpr int NBLK = SWIGLU ? 128 : 256;
+    constexpr int NDW = 4, NDT = 2;               // DMA instructions per wave and 128-k block: weights, tokens
+    // Operations that may stay in flight at the wait for a block: the DMA of the next block, NDW + NDT instructions
+    // (the counter retires in issue order).  The next block's two scale loads are issued before its DMA and are
+    // older still: not counting them costs at most a wait for two small loads that hit in L2, and keeps the count
+    // right for the first block, which has no scale loads of a block before it behind its DMA.
+    constexpr int VM_BLOCK = NDW + NDT;
+    static_assert(TG >= 1 && 16 * TG <= S8_TROWS, "token rows staged");
+    const int tid = threadIdx.x, lane = tid & 63, wave = uni(tid >> 6);
+    const int n0 = n_tile * NBLK;
+    const int K = g.K, N = g.N;
+    const int npair = K >> 7;
+    // N tile t walks k from 128-k block t (mod the number of blocks), so that the requests in flight on the chip do
+    // not share their low address bits (weight rows are K bytes apart); a column's order depends on its tile alone
+    const int prot = n_tile % npair;
+
+    // ---- DMA coordinates ----
+    // weights, instruction i: rows 8 i + lane / 8 of the wave's 32 (fragment i / 2, fragment row 8 (i & 1) + lane / 8)
+    const int lr = lane >> 3, pp = lane & 7;
+    uint32_t w_voff[NDW];
+    const uint8_t* bmat[2];
+    gptr_f32 sc[2];
+    int srow[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        bmat[j] = uni_ptr((SWIGLU && j == 1) ? g.b1[e] : g.b0[e]);
+        sc[j] = (gptr_f32)(uintptr_t)uni_ptr((SWIGLU && j == 1) ? g.s1[e] : g.s0[e]);
+        srow[j] = min((n0 + (SWIGLU ? 0 : 32 * wave)) >> 7, (N >> 7) - 1) * npair;
+    }
+#pragma unroll
+    for (int i = 0; i < NDW; ++i) {
+        const int fr = 8 * (i & 1) + lr;
+        const int rt = SWIGLU ? 16 * wave + fr : 32 * wave + 16 * (i >> 1) + fr;      // row of the tile's N range
+        w_voff[i] = (uint32_t)min(n0 + rt, N - 1) * (uint32_t)K + (uint32_t)((pp ^ wsw(fr)) << 4);
+    }
+    // tokens, instruction i: rows 8 wave + 4 i + lane / 16 of the 64 staged, chunk lane % 16.  Gathered rows go through
+    // one descriptor over x (a row_map entry outside x reads zeros), sorted rows through one that starts at the tile.
+    uint32_t t_voff[NDT];
+    const uint8_t* a_base = reinterpret_cast<const uint8_t*>(g.a) + (g.row_map ? (size_t)0 : (size_t)row0 * K * 2);
+    const int a_records = g.row_map ? (int)(uint32_t)g.a_bytes : -1;
+#pragma unroll
+    for (int i = 0; i < NDT; ++i) {
+        const int tr = 8 * wave + 4 * i + (lane >> 4);
+        const int r = min(row0 + tr, row_end - 1);
+        const int src = g.row_map ? ((gptr_i32)(uintptr_t)g.row_map)[r] : r - row0;
+        t_voff[i] = (uint32_t)src * (uint32_t)(K * 2) + (uint32_t)(((lane & 15) ^ tsw(tr)) << 4);
+        if (g.row_map && (unsigned)src >= (unsigned)g.a_rows) t_voff[i] = 0xfffffff0u;      // past any descriptor: zeros
+    }
+    float rsc[2][2];                              // block scales of the block being multiplied / of the next one
+    auto scales = [&](int p_pipe, int set) {
+        int pr = min(p_pipe, npair - 1) + prot;
+        pr = pr >= npair ? pr - npair : pr;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)(uintptr_t)sc[j], 0, -1, 0x00020000);
+            rsc[set][j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, 0, (srow[j] + pr) * 4, 0));
+        }
+    };
+    auto dma = [&](int p_pipe, uint8_t* buf) {
+        // past the end of k nobody reads what arrives: an empty descriptor returns zeros without touching memory,
+        // and the instruction still counts
+        const int live = uni(p_pipe < npair ? -1 : 0);   // (a scalar, or the descriptor ends up in vector registers)
+        int pr = min(p_pipe, npair - 1) + prot;
+        pr = pr >= npair ? pr - npair : pr;
+#pragma unroll
+        for (int i = 0; i < NDW; ++i) {
+            const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)bmat[i >> 1], 0, live, 0x00020000);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_u8)(buf + wave * 4096 + i * 1024), 16, w_voff[i], (uint32_t)(pr * 128), 0, 0);
+        }
+        const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)a_base, 0, live & a_records, 0x00020000);
+#pragma unroll
+        for (int i = 0; i < NDT; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_u8)(buf + S8_WBYTES + wave * 2048 + i * 1024), 16, t_voff[i],
+                                                     (uint32_t)(pr * 256), 0, 0);
+    };
+
+    const int frow = lane & 15, q = lane >> 4;
+    const uint32_t w_rd = (uint32_t)(wave * 4096 + frow * 128), wkey = (uint32_t)wsw(frow);
+    const uint32_t t_rd = (uint32_t)(S8_WBYTES + frow * 256), tkey = (uint32_t)tsw(frow);   // (group bases are multiples of 16)
+    f32x4 acc[TG][2];
+#pragma unroll
+    for (int t = 0; t < TG; ++t) { acc[t][0] = f32x4{0}; acc[t][1] = f32x4{0}; }
+
+    // Iteration p multiplies block p out of buffer p % 3.  Before it: this wave's DMA of block p has landed (at most the
+    // DMA of block p + 1 is outstanding) and its LDS reads have returned, then everybody's (a bare s_barrier: a fence
+    // would make the compiler wait for ALL outstanding DMA).  After the barrier every wave has left block p - 1,
+    // whose buffer takes block p + 2.  The scale loads come BEFORE the DMA: the compiler's own wait for a scale
+    // counts everything issued after it as allowed to be in flight.
+    auto iteration = [&](int p, const uint8_t* rd, uint8_t* refill, int sset) __attribute__((always_inline)) {
+        // (lgkmcnt: this wave's LDS reads of block p - 1 have returned -- its last matrix instructions may be scheduled
+        // behind the barrier, and the buffer they read is refilled right after it)
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" :: "n"(VM_BLOCK) : "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        scales(p + 1, sset ^ 1);
+        dma(p + 2, refill);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            bf16x8 wa[2][2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const u32x4 raw = *reinterpret_cast<const u32x4*>(rd + w_rd + j * 2048 + (((4 * h + q) ^ wkey) << 4));
+                wa[j][0] = __builtin_bit_cast(bf16x8, dequant8(raw[0], raw[1], rsc[sset][j]));
+                wa[j][1] = __builtin_bit_cast(bf16x8, dequant8(raw[2], raw[3], rsc[sset][j]));
+            }
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2) {
+                const uint32_t coff = (uint32_t)(((8 * h + 2 * q + s2) ^ tkey) << 4);
+#pragma unroll
+                for (int t = 0; t < TG; ++t) {
+                    const bf16x8 tf = *reinterpret_cast<const bf16x8*>(rd + t_rd + t * 16 * 256 + coff);
+                    acc[t][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[0][s2], tf, acc[t][0], 0, 0, 0);
+                    acc[t][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[1][s2], tf, acc[t][1], 0, 0, 0);
+                }
+            }
+        }
+    };
+    scales(0, 0);
+    dma(0, buf0);
+    dma(1, buf1);
+    int p = 0;
+    for (; p + 3 <= npair; p += 3) {
+        iteration(p, buf0, buf2, 0);
+        iteration(p + 1, buf1, buf0, 1);
+        iteration(p + 2, buf2, buf1, 0);
+        // (three iterations flip the scale set: swap so that the loop body keeps literal indices)
+        const float t0 = rsc[0][0], t1 = rsc[0][1];
+        rsc[0][0] = rsc[1][0]; rsc[0][1] = rsc[1][1];
+        rsc[1][0] = t0; rsc[1][1] = t1;
+    }
+    if (p < npair) {
+        iteration(p, buf0, buf2, 0);
+        if (p + 1 < npair) iteration(p + 1, buf1, buf0, 1);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no DMA may land in LDS after the workgroup has gone
+
+    // ---- epilogue: a lane holds 4 consecutive columns of one row per accumulator and stores them itself ----
+#pragma unroll
+    for (int t = 0; t < TG; ++t) {
+        const int r = row0 + 16 * t + frow;
+        if (r >= row_end) continue;
+        if (SWIGLU) {
+            const int col = n0 + 16 * wave + 4 * q;
+            if (col < N) *reinterpret_cast<u32x2*>(g.c + (size_t)r * N + col) = epilogue_pack<true>(acc[t][0], acc[t][1]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int col = n0 + 32 * wave + 16 * j + 4 * q;
+                if (col < N) *reinterpret_cast<u32x2*>(g.c + (size_t)r * N + col) = epilogue_pack<false>(acc[t][j], acc[t][j]);
+            }
+        }
+    }
+}
+
 // M tiles of an expert with `count` rows in the one-workgroup-per-tile kernel: one tile of 64, 128 or (bf16 weights)
 // 192 rows if that holds them all, else tiles of 128.  The height follows the EXPERT, not the launch: a tile taller
 // than its expert stages and multiplies rows that do not exist, and an expert cut into several tiles reads its
@@ -650,8 +836,10 @@ template <int WN, bool SWIGLU, bool W8>
 __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     constexpr int NT = 128 * WN;
     constexpr int STAGE_MAX = ((W8 ? 128 : 192) + BN_ROWS) * ROW_B;   // a stage of the tallest tile
-    __shared__ __attribute__((aligned(16))) uint8_t smem0[STAGE_MAX];
-    __shared__ __attribute__((aligned(16))) uint8_t smem1[STAGE_MAX];
+    __shared__ __attribute__((aligned(1024))) uint8_t smem0[STAGE_MAX];
+    __shared__ __attribute__((aligned(1024))) uint8_t smem1[STAGE_MAX];
+    __shared__ __attribute__((aligned(1024))) uint8_t smem2[W8 ? S8_BUF : 16];   // third buffer of the fp8 weight streamer
+    static_assert(!W8 || STAGE_MAX >= S8_BUF, "the streamer's buffers are the two stages and a third array");
     __shared__ int s_pref[MAX_E + 1];
     __shared__ int s_wtot[NT / 64];
     __shared__ int s_sel[5];
@@ -659,6 +847,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
 
     // ---- M-tile prefix over experts ----
     ExpertOfThread mine;
+    const bool s8_ok = !g.row_map || g.a_bytes < (1ull << 32);   // (the weight streamer addresses gathered rows with 32-bit offsets)
     int run = mtile_prefix_scan<NT>(g, tid, s_pref, s_wtot, mine, [&](int c) {
         if (g.rem_split) c &= 255;      // the rows the persistent kernel's full tiles leave over
         return c > g.cold_max ? 0 : tiles_of<(W8 ? 128 : 192)>(c);
@@ -721,6 +910,17 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     }
     const int row_end = uni(s_sel[4]);
     const int first_row = uni(s_sel[3]) + (g.rem_split ? ((row_end - uni(s_sel[3])) & ~255) : 0);
+    if (W8 && g.cold_max == 0x7fffffff && row_end - first_row <= 64 && s8_ok) {
+        // (this kernel has the call to itself, so no other kernel's summation order has to be matched.  An expert of
+        // 65 to 128 rows as two such tiles on neighbouring workgroups measured slower than one 128-row tile of
+        // gemm_tile: 2.99 against 3.68 TB/s of weights at 96 rows per expert.)
+        const int rows = row_end - first_row;
+        if (rows <= 16) stream8_tile<1, SWIGLU>(g, smem0, smem1, smem2, e, first_row, row_end, n_tile);
+        else if (rows <= 32) stream8_tile<2, SWIGLU>(g, smem0, smem1, smem2, e, first_row, row_end, n_tile);
+        else if (rows <= 48) stream8_tile<3, SWIGLU>(g, smem0, smem1, smem2, e, first_row, row_end, n_tile);
+        else stream8_tile<4, SWIGLU>(g, smem0, smem1, smem2, e, first_row, row_end, n_tile);
+        return;
+    }
     if (row_end - first_row <= 64) gemm_tile<1, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
     else if (row_end - first_row <= 128) gemm_tile<2, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
     else if (!W8 && mt_e == 1) gemm_tile<3, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
@@ -756,7 +956,6 @@ __device__ __forceinline__ int fresh_lane() {
 //    an outstanding DMA gets a vmcnt(0) in front of it; the fp8 weight stores must not.
 //  * stage parities are literals (the k loop is unrolled by two), so reads of one stage provably do not
 //    alias the DMA into the other.
-typedef __attribute__((address_space(3))) uint8_t* lds_u8;
 template <bool SWIGLU, bool W8>
 __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g) {
     constexpr int MT = 4, WN = 4;
@@ -905,12 +1104,19 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
         const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)((SWIGLU && i >= NB / 2) ? b8m1 : b8m0), 0, -1, 0x00020000);
         return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, b8_voff[i], kofs, 0));
     };
+    // Block scales come through buffer loads too, although their address is the same for every lane: as loads
+    // through a pointer the compiler would be free to make them scalar loads, and the hand-written vmcnt
+    // immediates below count them as vector-memory operations.
+    auto load_scale = [&](gptr_f32 sc, int idx) {
+        const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)(uintptr_t)sc, 0, -1, 0x00020000);
+        return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, 0, idx * 4, 0));
+    };
     auto gload_b = [&](int kt) {
         const size_t kofs = (size_t)kt * BK;
 #pragma unroll
         for (int i = 0; i < NB; ++i) rb[i] = load_b8(i, (uint32_t)kofs);
-        rs[0] = sc0[srow0 + (kt >> 1)];
-        rs[1] = sc1[srow1 + (kt >> 1)];
+        rs[0] = load_scale(sc0, srow0 + (kt >> 1));
+        rs[1] = load_scale(sc1, srow1 + (kt >> 1));
     };
     auto store_b_all = [&](uint8_t* Bs) {
 #pragma unroll
@@ -927,8 +1133,8 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
         *reinterpret_cast<u32x4*>(Bs + ((half ^ (b_swap ? 1 : 0)) ? b_lds[1] : b_lds[0]) + b * RB * ROW_B) = o;
         if (half == 1) {
             rb[b] = load_b8(b, (uint32_t)(kn * BK));
-            if (b / (NB / 2) == 0) rs[0] = sc0[srow0 + (kn >> 1)];
-            else rs[1] = sc1[srow1 + (kn >> 1)];
+            if (b / (NB / 2) == 0) rs[0] = load_scale(sc0, srow0 + (kn >> 1));
+            else rs[1] = load_scale(sc1, srow1 + (kn >> 1));
         }
     };
 
@@ -967,6 +1173,9 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
     // iteration kt multiplies stage par; the DMA brings k-stage ka (of the tile whose coordinates are current) into
     // the other token stage (and weight stage, bf16); fp8 converts the weight registers (k-stage kt+1) into the other
     // weight stage and refills them with k-stage kb
+    // Vector-memory operations a wave issues per k-iteration AFTER its DMA of the next stage; they may stay in flight
+    // at the iteration's barrier: the fp8 weight chunks (NB buffer loads) and their two block scales (buffer loads).
+    constexpr int VM_TAIL = W8 ? NB + 2 : 0;
     auto iteration = [&](int kt, int ka, int kb, int par) {
         const uint8_t* rdA = par ? sA1 : sA0; const uint8_t* rdB = par ? sB1 : sB0;
         uint8_t* wrA = par ? sA0 : sA1; uint8_t* wrB = par ? sB0 : sB1;
@@ -991,8 +1200,8 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        // this wave's DMA has landed (the four younger loads are the fp8 weight chunks and scales), then everybody's
-        if (W8) asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // this wave's DMA has landed (the younger loads are the fp8 weight chunks and scales), then everybody's
+        asm volatile("s_waitcnt vmcnt(%0)" :: "n"(VM_TAIL) : "memory");
         __syncthreads();
     };
     static_assert(NU == 8 && ND == 4 && (!W8 || NB == 2), "slot plan");
@@ -1005,10 +1214,8 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
         gload_b(0);
         store_b_all(sB0);
         gload_b(1);
-        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    } else {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(VM_TAIL) : "memory");   // (all but gload_b(1)'s NB + 2 loads)
     __syncthreads();
     constexpr int CW = SWIGLU ? 8 * TN : 16 * TN;    // output columns of this wave
     for (;;) {

@@ -217,6 +217,39 @@ def test_a_row_does_not_depend_on_its_place_in_its_expert(fp8, counts):
     assert torch.equal(y3, y2)
 
 
+@pytest.mark.parametrize("h,I", [(512, 384), (2048, 1024)])
+def test_fp8_weight_streamer_rows_do_not_depend_on_the_tile(h, I):
+    """fp8 experts of up to 64 rows, in a call below a mean of 128 rows per expert, go through the weight streamer
+    (weights by DMA as fp8, one 16/32/48/64-row body per expert).  Eight experts that share one set of weights and
+    hold 5 ... 64 rows, each starting with the same five rows: those rows come out bit-identical from every body,
+    against the oracle within the layer bound, and the call gives the same bits every time it runs (the buffers of
+    a tile are refilled while other waves still multiply; a missing wait shows as run-to-run differences)."""
+    from moe_gen_amd import ops
+    counts = [5, 16, 17, 32, 33, 48, 49, 64]
+    E = len(counts)
+    print(f"fp8 streamer h={h} I={I} counts={counts}", flush=True)
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    n = int(offsets[-1])
+    g = torch.Generator().manual_seed(97)
+    x = torch.randn(n, h, generator=g).to(torch.bfloat16)
+    for e in range(1, E):
+        x[offsets[e]:offsets[e] + 5] = x[:5]
+    one = make_experts(1, h, I, True, 98)[0]
+    dm = [tuple(t.cuda() for t in m) for m in one]
+    ptrs = ops.expert_pointers([dm[0][0]] * E, [dm[1][0]] * E, [dm[2][0]] * E, [dm[0][1]] * E, [dm[1][1]] * E, [dm[2][1]] * E)
+    off_d = torch.from_numpy(offsets).cuda()
+    xd = x.cuda()
+    ys = [ops.grouped_swiglu(xd, None, ptrs, off_d, n).clone() for _ in range(8)]
+    torch.cuda.synchronize()
+    for rep in range(1, 8):
+        assert torch.equal(ys[rep], ys[0]), f"call {rep} differs from call 0"
+    for e in range(1, E):
+        assert torch.equal(ys[0][offsets[e]:offsets[e] + 5], ys[0][:5]), f"expert {e} ({counts[e]} rows)"
+    wg, wu, wd = (f32_of(m) for m in one)
+    ref = O.mlp_f32(O.bf16_to_f32(bits(x)), wg, wu, wd)
+    assert rel_max(O.bf16_to_f32(bits(ys[0])), ref) <= TOL
+
+
 @pytest.mark.parametrize("fp8", [False, True])
 @pytest.mark.parametrize("E,mean", [(700, 3), (1024, 2), (600, 200), (400, 200)])
 def test_grouped_many_experts(fp8, E, mean):
