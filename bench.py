@@ -169,6 +169,76 @@ def staged_run(w, blk, x, steps: int, routing_aware: bool = False, pool: int = 0
             "note": note + "; bounded by the host link, not by the kernels"}
 
 
+def staged_host_run(w, steps: int = 20, pool: int = 0):
+    """Host-side cost of the staged path per layer call: a block with the workload's expert count and routing rules
+    but small matrices (hidden 512, intermediate 256) and 64 tokens, so that the kernels take next to nothing, its
+    experts behind an engine that hands out the RESIDENT weights (no copy, no PCIe) through the wrapper protocol
+    with the reference's pool size.  What is timed is the Python / ctypes work of walking the layer in waves:
+    get_weights / free_weights_buffer per expert, pointer tables and two grouped launches per wave (plus the one
+    read of the per-expert counts, which waits for the router and the dispatch)."""
+    import time as _t
+
+    import torch
+    import torch.nn as nn
+    from moe_gen_amd import StagedExpert, synthetic
+
+    w = w.scaled(n=64, h=512, I=256, seq=64)
+    blk = synthetic.build_block(w, device="cuda:0", gen_device="cuda:0")
+    names = blk.experts[0].names
+    has_shared = bool(w.S) and w.family != "mixtral"
+    n_slots = pool if pool > 0 else min(20, 2 * w.E)
+
+    class ResidentEngine:
+        stream_ordered_release = True
+
+        def __init__(self):
+            self.table = {}
+
+        def pool_size(self, module_type):
+            return n_slots if module_type == "routed_expert" else 1
+
+        def get_weights(self, key):
+            return self.table[key]
+
+        def free_weights_buffer(self, key):
+            pass
+
+        def clear_expert_buffer(self, layer_idx, expert_idx):
+            return 0
+
+    eng = ResidentEngine()
+
+    def scales_of(mlp):
+        return {f"{n}.weight_scale_inv": getattr(mlp, n).weight_scale_inv.data for n in names} if w.fp8 else None
+
+    L = 3
+    staged = []
+    for e, ex in enumerate(blk.experts):
+        eng.table[f"routed_expert_{L}_{e}"] = {f"{n}.weight": getattr(ex, n).weight.data for n in names}
+        staged.append(StagedExpert(ex, L, e, eng, scales_of(ex)))
+    sh = None
+    if has_shared:
+        eng.table[f"shared_expert_{L}"] = {f"{n}.weight": getattr(blk.shared_experts, n).weight.data for n in names}
+        sh = StagedExpert(blk.shared_experts, L, -1, eng, scales_of(blk.shared_experts))
+    x = synthetic.hidden_states(w, "cuda:0")
+    blk.experts = nn.ModuleList(staged)
+    if has_shared:
+        blk.shared_experts = sh
+    for _ in range(3):
+        blk(x)
+    torch.cuda.synchronize()
+    t0 = _t.perf_counter()
+    for _ in range(steps):
+        blk(x)
+    t_host = _t.perf_counter() - t0                 # the calls have returned: everything is enqueued
+    torch.cuda.synchronize()
+    t_all = _t.perf_counter() - t0
+    waves = -(-w.E // max(1, n_slots // 2)) if w.E > n_slots else 1
+    return {"host_ms_per_layer": t_host * 1e3 / steps, "wall_ms_per_layer": t_all * 1e3 / steps, "waves_per_layer": waves,
+            "pool_slots": n_slots, "tokens": 64, "hidden": w.h, "moe_intermediate": w.I,
+            "note": "engine hands out resident weights (no copies), small matrices: Python / ctypes cost of the wave walk per layer call"}
+
+
 def decoder_half_run(w, blk, x, steps: int):
     """The MLP half of a decoder layer around the block (post-attention RMSNorm, block, residual
     add): the library's fused form (one norm kernel, residual folded into the combine) against
@@ -420,6 +490,7 @@ def run_workload(name: str, args, with_cpu: bool):
         result["staged"] = staged_run(w, blk, x, max(2, args.steps // 2), pool=args.staged_pool)
         result["staged_routing_aware"] = staged_run(w, blk, x, max(2, args.steps // 2), routing_aware=True, pool=args.staged_pool)
         result["staged"]["pool_slots"] = result["staged_routing_aware"]["pool_slots"] = args.staged_pool or min(20, 2 * w.E)
+        result["staged_host"] = staged_host_run(w, pool=args.staged_pool)
     if with_cpu:
         # full size where the workload is small (DeepSeek-V2-Lite 4096 tokens, the 256-token decode case),
         # a bounded sample of the first tokens elsewhere
@@ -532,6 +603,7 @@ def main():
     ap.add_argument("--no-calibration", action="store_true", help="skip the vendor-dense / own-dense GEMM yardsticks")
     ap.add_argument("--staged", action="store_true", help="also time the block with weights staged from pinned host memory")
     ap.add_argument("--staged-pool", type=int, default=0, help="routed-expert slots of the staging pool (default 20, the reference engine's prefill default)")
+    ap.add_argument("--staged-host", action="store_true", help="only the host-side cost of the staged path per layer call")
     ap.add_argument("--decoder-half", action="store_true", help="also time RMSNorm + block + residual add, fused and separate")
     ap.add_argument("--cpu-sample", type=int, default=1024, help="tokens of the workload the CPU baseline runs")
     ap.add_argument("--ceiling", action="store_true", help="instead of the benchmark: registers-only MFMA rate, vendor dense "

@@ -128,6 +128,19 @@ def _tensors_of(expert, fetched=None):
     fetched: optional dict `"<proj>.weight" -> tensor` obtained from an engine's get_weights();
     block scales come from the Linear's `weight_scale_inv` or, for a wrapped expert, from the
     wrapper's `weight_dequant_scale["<proj>.weight_scale_inv"]` (Wrapper.py:482-489)."""
+    if fetched is not None:                     # hot path of the staged walk: no attribute look-ups on the modules
+        keys = expert.__dict__.get("_moe_keys")
+        if keys is None:                        # the tensor names of this expert, built once
+            names = _unwrap(expert).names
+            keys = (tuple(n + ".weight" for n in names), tuple(n + ".weight_scale_inv" for n in names))
+            expert.__dict__["_moe_keys"] = keys
+        wk, sk = keys
+        w0 = fetched[wk[0]]
+        if w0.dtype != FP8:
+            return (w0, fetched[wk[1]], fetched[wk[2]], None, None, None)
+        wrap_scales = expert.__dict__.get("weight_dequant_scale")
+        if wrap_scales:
+            return (w0, fetched[wk[1]], fetched[wk[2]], wrap_scales.get(sk[0]), wrap_scales.get(sk[1]), wrap_scales.get(sk[2]))
     mlp = _unwrap(expert)
     wrap_scales = getattr(expert, "weight_dequant_scale", None) or {}
     ws, ss = [], []
@@ -323,18 +336,23 @@ def _engine_experts(block, timer, tag, experts, a_rows, row_map, offsets, n_rows
         counts_host = counts.tolist()                        # one read of E integers (the reference reads them too, :673)
     hidden, inter = a_rows.shape[1], None
     act = y = None
+    stream = torch.cuda.current_stream().cuda_stream       # looked up once per layer call, not per wave
+    checked = False
 
     def launch(rows, a, b, rows_in_wave):
-        nonlocal act, y, inter
-        ptrs = _pointer_table(rows)
+        nonlocal act, y, inter, checked
+        ptrs = ops.expert_pointers_of_rows(rows, a_rows.device)
         if y is None:
             inter = ptrs.inter
             act = torch.empty((n_rows, inter), dtype=torch.bfloat16, device=a_rows.device)
             y = torch.empty((n_rows, hidden), dtype=torch.bfloat16, device=a_rows.device)
         bound = n_rows if rows_in_wave is None else rows_in_wave
+        if not 0 <= bound <= n_rows:
+            raise ValueError(f"rows of the wave {bound} outside [0, {n_rows}]")
         off = offsets[a:b + 1]
-        if timer is None:
-            ops.grouped_swiglu(a_rows, row_map, ptrs, off, n_rows, act, y, rows_bound=bound)
+        if timer is None:       # (the first wave validates the layer's buffers; the later ones pass the same)
+            ops.grouped_swiglu(a_rows, row_map, ptrs, off, n_rows, act, y, rows_bound=bound, checked=checked, stream=stream)
+            checked = True
         else:
             with timer.span(tag + "_gate_up"):
                 ops.grouped_swiglu(a_rows, row_map, ptrs, off, n_rows, act, y, ops.PHASE_GATE_UP, rows_bound=bound)

@@ -173,21 +173,115 @@ def expert_pointers(gates, ups, downs, s_gates=None, s_ups=None, s_downs=None, d
     return ExpertPointers(E, h, I, fp8, table(gates), table(ups), table(downs), sg, su, sd, keep)
 
 
+class _PinnedRing:
+    """A ring of small pinned host buffers for pointer tables on their way to the device: a table is written into
+    the next buffer and copied with one asynchronous H2D copy; a buffer is reused only after the copy that read it
+    last has completed (its event), which after a trip round the ring it long has."""
+
+    def __init__(self, n_buffers: int = 32, words: int = 8192):
+        self.bufs = [torch.empty(words, dtype=torch.int64, pin_memory=True) for _ in range(n_buffers)]
+        self.views = [b.numpy() for b in self.bufs]
+        self.events = [None] * n_buffers
+        self.i = 0
+        self.words = words
+
+    def push(self, values, device) -> torch.Tensor:
+        n = len(values)
+        if n > self.words:
+            return torch.tensor(values, dtype=torch.int64).to(device)
+        i = self.i
+        self.i = (i + 1) % len(self.bufs)
+        if self.events[i] is not None:
+            self.events[i].synchronize()
+        self.views[i][:n] = values
+        dev = torch.empty(n, dtype=torch.int64, device=device)
+        dev.copy_(self.bufs[i][:n], non_blocking=True)
+        ev = self.events[i] or torch.cuda.Event()
+        ev.record()
+        self.events[i] = ev
+        return dev
+
+
+_rings: dict = {}
+_table_cache: dict = {}       # (device, shape, dtype, pointers) -> ExpertPointers of a wave seen before
+_TABLE_CACHE_MAX = 32768
+
+
+def expert_pointers_of_rows(rows, device) -> ExpertPointers:
+    """Pointer tables for one wave of engine-delivered experts: `rows[i]` = (gate, up, down[, s_gate, s_up, s_down])
+    of expert i.  The hot form of expert_pointers: shapes and dtypes are checked against the first expert's, all
+    tables travel in ONE pinned, asynchronous copy (six synchronous ones otherwise: 26 waves of a DeepSeek-V3 layer
+    cost 2.4 ms of host time that way), and the tables are slices of that one device array."""
+    E = len(rows)
+    g0, u0, d0 = rows[0][0], rows[0][1], rows[0][2]
+    I, h = g0.shape
+    fp8 = g0.dtype == torch.float8_e4m3fn
+    want = torch.float8_e4m3fn if fp8 else torch.bfloat16
+    gs, ds = (I, h), (h, I)
+    if not g0.is_cuda:
+        raise RuntimeError(f"expert weights must live on the GPU (got {g0.device}); this package has no CPU path")
+    ncol = 6 if fp8 else 3
+    vals = []
+    for c in range(ncol):
+        for r in rows:
+            vals.append(r[c].data_ptr())
+    # Slot addresses recur from call to call (an engine's pool is a fixed set of buffers, block scales are
+    # resident): a wave whose pointers were all seen before, for tensors of this shape, reuses its device table.
+    ckey = (str(device), I, h, fp8, tuple(vals))
+    hit = _table_cache.get(ckey)
+    if hit is not None:
+        return hit
+    for i, r in enumerate(rows):
+        if r[0].shape != gs or r[1].shape != gs or r[2].shape != ds or r[0].dtype != want or r[1].dtype != want or r[2].dtype != want:
+            raise ValueError(f"experts[{i}]: weights must be {want} of shapes {gs}, {gs}, {ds}")
+        if fp8 and (r[3] is None or r[4] is None or r[5] is None):
+            raise ValueError("fp8 expert weights need their *_scale_inv block scales")
+    if fp8:
+        bi, bh = -(-I // 128), -(-h // 128)
+        for i, r in enumerate(rows):
+            if r[3].shape != (bi, bh) or r[4].shape != (bi, bh) or r[5].shape != (bh, bi) or r[3].dtype != torch.float32:
+                raise ValueError(f"experts[{i}]: block scales must be fp32 of shapes {(bi, bh)}, {(bi, bh)}, {(bh, bi)}")
+    key = str(device)
+    ring = _rings.get(key)
+    if ring is None:
+        ring = _rings[key] = _PinnedRing()
+    t = ring.push(vals, device)
+    cols = [t[c * E:(c + 1) * E] for c in range(ncol)]
+    out = ExpertPointers(E, h, I, fp8, cols[0], cols[1], cols[2], *(cols[3:] if fp8 else (None, None, None)))
+    if len(_table_cache) >= _TABLE_CACHE_MAX:
+        _table_cache.clear()
+    _table_cache[ckey] = out       # (holds the device table only; the weights stay the engine's)
+    return out
+
+
 PHASE_GATE_UP, PHASE_DOWN, PHASE_BOTH = 1, 2, 3
 
 
 def grouped_swiglu(x: torch.Tensor, row_map, ptrs: ExpertPointers, offsets: torch.Tensor, n_rows: int,
                    act: torch.Tensor | None = None, y: torch.Tensor | None = None, phases: int = PHASE_BOTH,
-                   rows_bound: int | None = None):
+                   rows_bound: int | None = None, checked: bool = False, stream: int | None = None):
     """All experts' SwiGLU MLPs on their row ranges.  x: bf16 sorted rows [n_rows,h], or the
     unsorted matrix with row_map int32 [n_rows].  Returns y bf16 [n_rows,h] (sorted-row order).
 
     `ptrs` and `offsets` may describe a sub-range of a layer's experts (offsets = a slice
     offsets[a:b+1] of the layer's, absolute sorted rows): x, row_map, act and y stay the layer's
     full buffers, and rows_bound, if known, is the number of rows inside the range (it sizes the
-    launch and picks the tile shape; default: n_rows)."""
-    _need(x, torch.bfloat16, "x")
+    launch and picks the tile shape; default: n_rows).
+    checked / stream: a caller that walks one layer in many waves passes the same x, row_map, act and y every
+    time; it validates them on the first wave, says so, and passes the stream it looked up once."""
     h, I, E = ptrs.hidden, ptrs.inter, ptrs.n_experts
+    if checked:
+        if offsets.shape[0] != E + 1:
+            raise ValueError(f"offsets must have {E + 1} entries, got {offsets.shape[0]}")
+        if rows_bound is not None:
+            n_rows = rows_bound
+        st = _stream() if stream is None else stream
+        fn = N.lib().moe_grouped_swiglu_w8a16 if ptrs.fp8 else N.lib().moe_grouped_swiglu_bf16
+        scales = (_ptr(ptrs.s_gate), _ptr(ptrs.s_up), _ptr(ptrs.s_down)) if ptrs.fp8 else ()
+        N.check(fn(x.data_ptr(), x.shape[0], _ptr(row_map), _ptr(ptrs.w_gate), _ptr(ptrs.w_up), _ptr(ptrs.w_down), *scales,
+                   offsets.data_ptr(), n_rows, E, h, I, act.data_ptr(), y.data_ptr(), phases, None, 0, st), "moe_grouped_swiglu")
+        return y
+    _need(x, torch.bfloat16, "x")
     if x.shape[1] != h:
         raise ValueError(f"x has hidden size {x.shape[1]}, experts expect {h}")
     if row_map is None and x.shape[0] < n_rows:

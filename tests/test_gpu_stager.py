@@ -136,23 +136,35 @@ class ExpertWrapperLike(torch.nn.Module):
                                    else f"shared_expert_{layer_idx}")
 
 
-@pytest.mark.parametrize("name,n_slots", [("deepseek_v3_w8a16", 20), ("deepseek_v2_236b", 20), ("deepseek_v3_w8a16", 256),
-                                          ("deepseek_v2_236b", 7)])
-def test_block_with_engine_backed_experts(name, n_slots):
+@pytest.mark.parametrize("name,n_slots,phase,resident", [
+    ("deepseek_v3_w8a16", 20, "prefill", ()), ("deepseek_v2_236b", 20, "prefill", ()), ("deepseek_v3_w8a16", 256, "prefill", ()),
+    ("deepseek_v2_236b", 7, "prefill", ()),
+    ("mixtral_8x7b", 8, "prefill", ()), ("mixtral_8x7b", 3, "prefill", ()),           # pool = E and pool < E
+    ("deepseek_v3_w8a16", 20, "decoding", ()), ("mixtral_8x7b", 3, "decoding", ()),  # the decoding pool is the one that counts
+    ("deepseek_v2_236b", 7, "prefill", (0, 5, 6, 159)), ("mixtral_8x7b", 3, "prefill", (2, 7)),   # some experts stay resident
+])
+def test_block_with_engine_backed_experts(name, n_slots, phase, resident):
     """The block fed through MoE-Gen's expert-wrapper protocol against an engine with the
     reference's default pool of 20 routed-expert slots (deepseekv3_initializer.py:912-916), far
     fewer than the layer's experts: same bits as with resident weights, parity with the oracle,
-    never more than the pool held, one get/free per expert."""
+    never more than the pool held, one get/free per expert.  Mixtral's experts are wrapped the same
+    way (Mixtral_Initializer.py:761-787; w1 / w3 / w2, no shared expert).  In the decoding phase
+    (Expert_Wrapper.phase == "decoding", Wrapper.py:434) the pool size is read from
+    num_decoding_module_buffer (deepseekv3_initializer.py:918-927): the engine here then has that many
+    slots and a prefill entry that would be wrong.  `resident`: experts the initializer left out of the
+    copy task keep their weights and get_weights = False (deepseekv3_initializer.py:1259-1266)."""
     from types import SimpleNamespace as NS
     from moe_gen_amd import synthetic
     w = synthetic.WORKLOADS[name].scaled(n=256, h=512, I=256, seq=64)
-    print(f"engine-backed {name} pool {n_slots} of {w.E} experts", flush=True)
+    print(f"engine-backed {name} pool {n_slots} of {w.E} experts, phase {phase}, resident {resident}", flush=True)
     blk = synthetic.build_block(w, device="cuda", gen_device="cpu")
     x_cpu = synthetic.hidden_states(w, "cpu")
     x = x_cpu.cuda()
-    ref = blk(x).clone()
-    resident = synthetic.build_block(w, device="cuda", gen_device="cpu")     # keeps the weights for the oracle
+    first = lambda o: o[0] if isinstance(o, tuple) else o
+    ref = first(blk(x)).clone()
+    resident_blk = synthetic.build_block(w, device="cuda", gen_device="cpu")     # keeps the weights for the oracle
     names = blk.experts[0].names
+    has_shared = w.family != "mixtral"
     L = 7
     weights, wrapped = {}, []
 
@@ -163,24 +175,35 @@ def test_block_with_engine_backed_experts(name, n_slots):
             getattr(mlp, n).weight.data = torch.zeros(1, dtype=torch.bfloat16, device="cuda")
         return scales
 
-    scales = [detach(ex, f"routed_expert_{L}_{e}") for e, ex in enumerate(blk.experts)]
-    sscale = detach(blk.shared_experts, f"shared_expert_{L}")
+    scales = [None if e in resident else detach(ex, f"routed_expert_{L}_{e}") for e, ex in enumerate(blk.experts)]
+    sscale = detach(blk.shared_experts, f"shared_expert_{L}") if has_shared else None
     eng = FakeCoreEngine(weights, {"routed_expert": n_slots, "shared_expert": 1})
-    cfg = NS(GPU_Buffer_Config=NS(num_prefill_module_buffer={"routed_expert": n_slots, "shared_expert": 1},
-                                  num_decoding_module_buffer={"routed_expert": 4 * n_slots, "shared_expert": 1}))
+    in_phase = {"routed_expert": n_slots, "shared_expert": 1}
+    other = {"routed_expert": 4 * n_slots if phase == "prefill" else 1, "shared_expert": 1}
+    cfg = NS(GPU_Buffer_Config=NS(num_prefill_module_buffer=in_phase if phase == "prefill" else other,
+                                  num_decoding_module_buffer=other if phase == "prefill" else in_phase))
+
+    class Wrapper(ExpertWrapperLike):                     # `phase` is a class attribute of Expert_Wrapper (Wrapper.py:434)
+        pass
+
+    Wrapper.phase = phase
     for e, ex in enumerate(blk.experts):
-        wrapped.append(ExpertWrapperLike(ex, L, e, eng, scales[e], cfg))
+        wr = Wrapper(ex, L, e, eng, scales[e], cfg)
+        wr.get_weights = e not in resident
+        wrapped.append(wr)
     blk.experts = torch.nn.ModuleList(wrapped)
-    blk.shared_experts = ExpertWrapperLike(blk.shared_experts, L, -1, eng, sscale, cfg)
+    if has_shared:
+        blk.shared_experts = Wrapper(blk.shared_experts, L, -1, eng, sscale, cfg)
     for rep in range(2):                                  # the second call starts from a pool in mid-cycle
-        out = blk(x)
+        out = first(blk(x))
         torch.cuda.synchronize()
         assert torch.equal(out, ref), rep
-    check_against_oracle(resident, w, x_cpu, out, blk)
+    check_against_oracle(resident_blk, w, x_cpu, out, blk)
     assert eng.max_held <= max(n_slots, 1) and not eng.held
     gets = [c[1] for c in eng.calls if c[0] == "get"]
     frees = [c[1] for c in eng.calls if c[0] == "free"]
     assert sorted(gets) == sorted(frees) == sorted(list(weights) * 2)
+    assert not any(f"routed_expert_{L}_{e}" in gets for e in resident)
     assert ("clear", L, 0) in eng.calls
 
 
