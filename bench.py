@@ -81,14 +81,17 @@ def cpu_baseline(w, blk, n_sample: int, passes: int = 3):
                       "stock-PyTorch CPU restatement of the reference block"}
 
 
-def staged_run(w, blk, x, steps: int, routing_aware: bool = False, pool: int = 0):
+def staged_run(w, blk, x, steps: int, routing_aware: bool = False, pool: int = 0, pageable: bool = False):
     """Second figure: the same block with every expert matrix in pinned host memory, delivered by
     the stager (cyclic prefetch on the copy stream, event hand-off) into a pool of `pool` slots while
     earlier experts are multiplied.  Three layers' worth of modules take turns, as in a model (with two, the
     layer before the current one is also the next one, and the engine's rule that drops what is left of the
     previous layer would throw away what it has just prefetched whenever the pool holds two layers).
     routing_aware: copy only the experts that received tokens, busiest first, once the per-expert
-    counts are known (fewer bytes, but the copies cannot start before the router has run)."""
+    counts are known (fewer bytes, but the copies cannot start before the router has run).
+    pageable: the host copies of the weights are ORDINARY memory (a mapped weight segment that was not
+    allocated pinned) and travel through the stager's ring of 8 pinned chunks of 32 MiB, filled by 8 host
+    threads: the host holds the model once instead of twice."""
     import time as _t
 
     import torch
@@ -106,7 +109,8 @@ def staged_run(w, blk, x, steps: int, routing_aware: bool = False, pool: int = 0
         shapes["shared_expert"] = {f"{n}.weight": (tuple(getattr(blk.shared_experts, n).weight.shape), wdt) for n in names}
         n_slots["shared_expert"] = 2
     st = Stager(shapes, n_slots, device="cuda:0", model_type={"v3": "deepseek_v3", "v2": "deepseek_v2"}.get(w.family, "mixtral"),
-                num_hidden_layers=64, num_local_experts=E)
+                num_hidden_layers=64, num_local_experts=E, bounce_chunks=8 if pageable else 0, bounce_chunk_bytes=32 << 20,
+                bounce_threads=8)
     layers = (10, 11, 12)
     if routing_aware:
         st.set_policy("routed_expert", "on_demand")
@@ -118,15 +122,16 @@ def staged_run(w, blk, x, steps: int, routing_aware: bool = False, pool: int = 0
 
     staged = {}
     host = {}
+    keep = (lambda t: t) if pageable else (lambda t: t.pin_memory())
     for e in range(E):
-        host[e] = {f"{n}.weight": getattr(blk.experts[e], n).weight.data.cpu().pin_memory() for n in names}
+        host[e] = {f"{n}.weight": keep(getattr(blk.experts[e], n).weight.data.cpu()) for n in names}
     if has_shared:
-        host["s"] = {f"{n}.weight": getattr(blk.shared_experts, n).weight.data.cpu().pin_memory() for n in names}
+        host["s"] = {f"{n}.weight": keep(getattr(blk.shared_experts, n).weight.data.cpu()) for n in names}
     for L in layers:
         for e in range(E):
-            st.add_module(f"routed_expert_{L}_{e}", "routed_expert", host[e])
+            st.add_module(f"routed_expert_{L}_{e}", "routed_expert", host[e], pageable=pageable)
         if has_shared:
-            st.add_module(f"shared_expert_{L}", "shared_expert", host["s"])
+            st.add_module(f"shared_expert_{L}", "shared_expert", host["s"], pageable=pageable)
         staged[L] = ([StagedExpert(blk.experts[e], L, e, st, scales_of(blk.experts[e])) for e in range(E)],
                      StagedExpert(blk.shared_experts, L, -1, st, scales_of(blk.shared_experts)) if has_shared else None)
     resident_experts = blk.experts
@@ -163,9 +168,11 @@ def staged_run(w, blk, x, steps: int, routing_aware: bool = False, pool: int = 0
     st.close()
     note = ("only experts with a non-zero token count are staged, busiest first, after the router has run"
             if routing_aware else
+            "all expert weights re-staged from ordinary (pageable) host memory every step through 8 pinned chunks of 32 MiB"
+            if pageable else
             "all expert weights re-staged from pinned host memory every step (the reference's policy)")
     return {"tokens_per_s": w.n * steps / dt, "ms_per_step": dt * 1e3 / steps,
-            "host_to_hbm_gib_per_step": per_step / 2 ** 30,
+            "host_to_hbm_gib_per_step": per_step / 2 ** 30, "host_to_hbm_gbps": per_step / (dt / steps) / 1e9,
             "note": note + "; bounded by the host link, not by the kernels"}
 
 
@@ -489,6 +496,7 @@ def run_workload(name: str, args, with_cpu: bool):
     if args.staged:
         result["staged"] = staged_run(w, blk, x, max(2, args.steps // 2), pool=args.staged_pool)
         result["staged_routing_aware"] = staged_run(w, blk, x, max(2, args.steps // 2), routing_aware=True, pool=args.staged_pool)
+        result["staged_from_pageable_memory"] = staged_run(w, blk, x, max(2, args.steps // 2), pool=args.staged_pool, pageable=True)
         result["staged"]["pool_slots"] = result["staged_routing_aware"]["pool_slots"] = args.staged_pool or min(20, 2 * w.E)
         result["staged_host"] = staged_host_run(w, pool=args.staged_pool)
     if with_cpu:

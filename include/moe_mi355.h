@@ -308,6 +308,21 @@ int moe_stage_create(moe_stager** out, int32_t n_types, const size_t* slot_bytes
  * to back into the slot at dst_offsets.  Returns the module id (>= 0). */
 int moe_stage_add_module(moe_stager* s, int32_t type, int32_t n_tensors,
                          const void* const* src, const size_t* bytes, const size_t* dst_offsets);
+/*
+ * Sources in ORDINARY (pageable) host memory.  Weights_Storage::Init maps the reference's POSIX shm weight
+ * segment once and views it (core/Weights_Storage/Weights_Storage.cpp:52-78, core/Parameter_Server/posix_shm.cpp:36-92),
+ * registering the mapping with the GPU runtime; this library never registers existing memory.  Instead of a second,
+ * pinned copy of the whole model, modules registered with moe_stage_add_module_pageable (or
+ * moe_stage_add_module_from_segment) travel through a ring of n_chunks pinned chunks of chunk_bytes each, allocated
+ * here: a worker thread copies a piece into the next chunk with n_threads host threads and enqueues the
+ * hipMemcpyAsync out of it, refilling a chunk once its previous transfer has completed.  Pinned memory held:
+ * n_chunks * chunk_bytes.  moe_stage_acquire of such a module blocks the calling host thread until the worker has
+ * enqueued the module's transfers (as the reference's get_weights waits for its copy worker); the stream hand-off
+ * by events is unchanged.  Call once, before the first copy of a pageable module.
+ */
+int moe_stage_set_bounce(moe_stager* s, int32_t n_chunks, size_t chunk_bytes, int32_t n_threads);
+int moe_stage_add_module_pageable(moe_stager* s, int32_t type, int32_t n_tensors,
+                                  const void* const* src, const size_t* bytes, const size_t* dst_offsets);
 /* Issue copies for the next modules of every type while free slots exist
  * (one turn of the reference's worker loop per free slot).  Returns the number
  * of modules whose copy was enqueued. */
@@ -417,6 +432,15 @@ int moe_stage_add_module_from_arena(moe_stager* s, int32_t type, const moe_arena
                                     const char* module_key, const void* arena_base,
                                     size_t arena_bytes, int32_t n_tensors,
                                     const char* const* tensor_keys, const size_t* dst_offsets);
+/*
+ * The same for a segment in ordinary (pageable) host memory -- the mapped shm weight segment itself, not a pinned
+ * copy of it (Weights_Storage.cpp:52-78, posix_shm.cpp:36-92): the module's copies go through the stager's bounce
+ * ring (moe_stage_set_bounce), so the host holds the model once.
+ */
+int moe_stage_add_module_from_segment(moe_stager* s, int32_t type, const moe_arena_index* ix,
+                                      const char* module_key, const void* segment_base,
+                                      size_t segment_bytes, int32_t n_tensors,
+                                      const char* const* tensor_keys, const size_t* dst_offsets);
 
 #ifdef __cplusplus
 }

@@ -68,6 +68,12 @@ SIGNATURES = {
     "moe_stage_add_module_from_arena": (ctypes.c_int, [c_void_p, c_int32, c_void_p, ctypes.c_char_p, c_void_p, c_size_t,
                                                        c_int32, ctypes.POINTER(ctypes.c_char_p),
                                                        ctypes.POINTER(c_size_t)]),
+    "moe_stage_add_module_from_segment": (ctypes.c_int, [c_void_p, c_int32, c_void_p, ctypes.c_char_p, c_void_p, c_size_t,
+                                                         c_int32, ctypes.POINTER(ctypes.c_char_p),
+                                                         ctypes.POINTER(c_size_t)]),
+    "moe_stage_set_bounce": (ctypes.c_int, [c_void_p, c_int32, c_size_t, c_int32]),
+    "moe_stage_add_module_pageable": (ctypes.c_int, [c_void_p, c_int32, c_int32, ctypes.POINTER(c_void_p),
+                                                     ctypes.POINTER(c_size_t), ctypes.POINTER(c_size_t)]),
     "moe_stage_create": (ctypes.c_int, [ctypes.POINTER(c_void_p), c_int32, ctypes.POINTER(c_size_t),
                                         ctypes.POINTER(c_int32), ctypes.POINTER(c_void_p), c_int32]),
     "moe_stage_set_policy": (ctypes.c_int, [c_void_p, c_int32, c_int32]),

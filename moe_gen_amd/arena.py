@@ -4,8 +4,10 @@ module_key -> tensor_key -> {offset, shape, byte_size} map (Parameter_Server.h:4
 Weights_Storage.cpp:52-77), in the reference's wire format (posix_shm.cpp:167-357).
 
 The reference maps a POSIX shm segment and registers it with the GPU runtime
-(posix_shm.cpp allocate_shared_pinned_memory).  Here the arena is ALLOCATED pinned
-(torch pin_memory=True) and filled by copy: registering existing memory is not supported."""
+(posix_shm.cpp allocate_shared_pinned_memory).  Registering existing memory is not supported
+here, so an arena is either ALLOCATED pinned and filled by copy (`pack`, `from_bytes`: a second
+copy of the weights in host memory), or left where it is, in ordinary memory, and streamed
+through the stager's small ring of pinned chunks (`stream_from`: the host holds the model once)."""
 from __future__ import annotations
 
 import ctypes
@@ -82,10 +84,22 @@ class Arena:
     """A pinned host buffer + its index.  `pack` lays tensors out back to back (256-byte aligned);
     `from_bytes` adopts an index and a data blob produced elsewhere (another process, a file)."""
 
-    def __init__(self, index: ArenaIndex, data: torch.Tensor):
+    def __init__(self, index: ArenaIndex, data: torch.Tensor, pageable: bool = False):
         if data.dtype != torch.uint8 or data.dim() != 1 or data.is_cuda or not data.is_contiguous():
             raise RuntimeError("arena data must be a contiguous 1-D uint8 host tensor")
-        self.index, self.data = index, data
+        self.index, self.data, self.pageable = index, data, pageable
+
+    @classmethod
+    def stream_from(cls, index_bytes: bytes, segment) -> "Arena":
+        """Adopt a weight segment WHERE IT LIES, in ordinary (pageable) host memory -- e.g. the
+        reference's shm segment mapped into this process (Weights_Storage.cpp:52-78,
+        posix_shm.cpp:36-92), as a uint8 tensor over the mapping (torch.from_numpy(np.memmap(...))
+        or torch.frombuffer).  Nothing is copied here: a Stager built with a bounce ring moves each
+        module through a few pinned chunks on its way to HBM, so the host holds the weights once
+        (from_bytes holds them twice: ~640 GB more for the DeepSeek-R1 checkpoint)."""
+        ix = ArenaIndex.parse(index_bytes)
+        data = segment if isinstance(segment, torch.Tensor) else torch.frombuffer(segment, dtype=torch.uint8)
+        return cls(ix, data.reshape(-1), pageable=True)
 
     @classmethod
     def pack(cls, modules: dict, pin: bool = True) -> "Arena":

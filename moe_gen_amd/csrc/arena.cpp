@@ -224,12 +224,11 @@ extern "C" int moe_arena_index_tensor(const moe_arena_index* ix, int32_t i, int3
 // Registers module `module_key` of the index with a stager: its tensors become copy sources at
 // arena_base + offset (Weights_Storage::Init, Weights_Storage.cpp:69-76).  tensor_keys[i] goes to
 // dst_offsets[i] of the slot; every listed tensor must exist and lie inside the arena.
-extern "C" int moe_stage_add_module_from_arena(moe_stager* st, int32_t type, const moe_arena_index* ix,
-                                               const char* module_key, const void* arena_base, size_t arena_bytes,
-                                               int32_t n_tensors, const char* const* tensor_keys,
-                                               const size_t* dst_offsets) {
+static int add_module_from(moe_stager* st, int32_t type, const moe_arena_index* ix, const char* module_key,
+                           const void* arena_base, size_t arena_bytes, int32_t n_tensors, const char* const* tensor_keys,
+                           const size_t* dst_offsets, bool pageable) {
     MOE_REQUIRE(st && ix && module_key && arena_base && tensor_keys && dst_offsets,
-                "moe_stage_add_module_from_arena: NULL argument");
+                "moe_stage_add_module_from_arena / _segment: NULL argument");
     MOE_REQUIRE(n_tensors >= 1 && n_tensors <= 64, "moe_stage_add_module_from_arena: n_tensors %d outside [1,64]",
                 n_tensors);
     auto it = ix->by_key.find(module_key);
@@ -256,5 +255,23 @@ extern "C" int moe_stage_add_module_from_arena(moe_stager* st, int32_t type, con
         src[i] = static_cast<const char*>(arena_base) + t.offset;
         bytes[i] = (size_t)t.byte_size;
     }
-    return moe_stage_add_module(st, type, n_tensors, src, bytes, dst_offsets);
+    return pageable ? moe_stage_add_module_pageable(st, type, n_tensors, src, bytes, dst_offsets)
+                    : moe_stage_add_module(st, type, n_tensors, src, bytes, dst_offsets);
+}
+
+extern "C" int moe_stage_add_module_from_arena(moe_stager* st, int32_t type, const moe_arena_index* ix,
+                                               const char* module_key, const void* arena_base, size_t arena_bytes,
+                                               int32_t n_tensors, const char* const* tensor_keys,
+                                               const size_t* dst_offsets) {
+    return add_module_from(st, type, ix, module_key, arena_base, arena_bytes, n_tensors, tensor_keys, dst_offsets, false);
+}
+
+// The same for a segment in ordinary (pageable) host memory, e.g. the reference's POSIX shm weight segment mapped
+// into this process (posix_shm.cpp:36-92) without a second, pinned copy of the model: the module's copies go
+// through the stager's bounce ring (moe_stage_set_bounce).
+extern "C" int moe_stage_add_module_from_segment(moe_stager* st, int32_t type, const moe_arena_index* ix,
+                                                 const char* module_key, const void* segment_base, size_t segment_bytes,
+                                                 int32_t n_tensors, const char* const* tensor_keys,
+                                                 const size_t* dst_offsets) {
+    return add_module_from(st, type, ix, module_key, segment_base, segment_bytes, n_tensors, tensor_keys, dst_offsets, true);
 }

@@ -23,9 +23,13 @@
 //   GPU_Weight_Buffer::clear_expert_buffer    GPU_Weight_Buffer.cpp:261-308  (moe_stage_clear_expert_buffer)
 //   MoE_Gen::set_phase -> resize_buffer       MoE_Gen.cpp:128-134            (moe_stage_set_phase)
 //   MoE_Gen::reset_prefill_buffer / reset_weight_copy_queue   MoE_Gen.cpp:205-211
+#include <condition_variable>
+#include <cstdlib>
 #include <cstring>
 #include <deque>
 #include <mutex>
+#include <string>
+#include <thread>
 #include <vector>
 
 #include "common.h"
@@ -45,6 +49,8 @@ struct Module {
     bool wanted = false;         // named by a fetch and not yet released (on-demand staging)
     int layer = -1, expert = -2; // tag: routed expert `expert` (>= 0) or shared expert (-1) of `layer`; -2 untagged
     hipEvent_t ready = nullptr;  // copy finished (device backend)
+    bool pageable = false;       // sources are ordinary host memory: copies go through the pinned bounce ring
+    uint64_t job_seq = 0;        // sequence number of this module's latest bounce job
 };
 
 struct Type {
@@ -60,10 +66,117 @@ struct Type {
     int n_prefill = 0, n_decoding = 0;  // slots per phase (0: the phase verbs leave this type alone)
 };
 
+// Copies out of PAGEABLE host memory (a mapped weight segment that was not allocated pinned): a worker thread
+// moves each module through a ring of pinned chunks -- host memcpy into the next chunk (split over a few helper
+// threads), then hipMemcpyAsync out of it on the copy stream -- so the segment is never copied whole and the
+// pinned memory is n_chunks x chunk_bytes.  A chunk is refilled once the event recorded behind its last
+// hipMemcpyAsync has completed; the memcpy into one chunk overlaps the DMA out of the others.
+struct BounceJob {
+    uint64_t seq = 0;
+    uint8_t* dst = nullptr;
+    std::vector<Piece> pieces;
+    hipEvent_t wait_for = nullptr;   // release event of the slot's previous user (device backend), or null
+    hipEvent_t ready = nullptr;
+};
+
+struct Bounce {
+    int n_chunks = 0, n_threads = 1, device = 0, backend = MOE_STAGE_DEVICE;
+    size_t chunk_bytes = 0;
+    hipStream_t stream = nullptr;
+    std::vector<uint8_t*> chunk;
+    std::vector<hipEvent_t> done;
+    std::vector<char> busy;
+    int next = 0;
+    std::thread worker;
+    std::mutex mu;
+    std::condition_variable cv_job, cv_done;
+    std::deque<BounceJob> jobs;
+    uint64_t enqueued = 0, issued = 0;   // jobs handed in / jobs whose copies have all been enqueued on the stream
+    bool stop = false;
+    int err = MOE_OK;
+    std::string err_msg;
+
+    void copy_in(uint8_t* dst, const uint8_t* src, size_t n) {   // pageable -> pinned, on n_threads threads
+        const size_t min_part = 1u << 20;
+        int parts = (int)std::min<size_t>((size_t)n_threads, (n + min_part - 1) / min_part);
+        if (parts <= 1) { std::memcpy(dst, src, n); return; }
+        std::vector<std::thread> th;
+        const size_t per = ((n / parts) + 4095) & ~(size_t)4095;
+        for (int i = 1; i < parts; ++i) {
+            const size_t a = std::min(n, per * i), b = std::min(n, per * (i + 1));
+            if (b > a) th.emplace_back([=] { std::memcpy(dst + a, src + a, b - a); });
+        }
+        std::memcpy(dst, src, std::min(n, per));
+        for (auto& t : th) t.join();
+    }
+    int run_job(const BounceJob& j) {
+        const bool dev = backend == MOE_STAGE_DEVICE;
+        if (dev && j.wait_for) MOE_HIP_CHECK(hipStreamWaitEvent(stream, j.wait_for, 0));
+        for (const Piece& p : j.pieces)
+            for (size_t off = 0; off < p.bytes; off += chunk_bytes) {
+                const size_t len = std::min(chunk_bytes, p.bytes - off);
+                const int c = next;
+                next = (next + 1) % n_chunks;
+                if (dev && busy[c]) MOE_HIP_CHECK(hipEventSynchronize(done[c]));
+                copy_in(chunk[c], static_cast<const uint8_t*>(p.src) + off, len);
+                if (dev) {
+                    MOE_HIP_CHECK(hipMemcpyAsync(j.dst + p.dst_off + off, chunk[c], len, hipMemcpyHostToDevice, stream));
+                    MOE_HIP_CHECK(hipEventRecord(done[c], stream));
+                    busy[c] = 1;
+                } else {
+                    std::memcpy(j.dst + p.dst_off + off, chunk[c], len);
+                }
+            }
+        if (dev) MOE_HIP_CHECK(hipEventRecord(j.ready, stream));
+        return MOE_OK;
+    }
+    void loop() {
+        if (backend == MOE_STAGE_DEVICE) (void)hipSetDevice(device);
+        for (;;) {
+            BounceJob j;
+            {
+                std::unique_lock<std::mutex> lk(mu);
+                cv_job.wait(lk, [&] { return stop || !jobs.empty(); });
+                if (jobs.empty()) return;
+                j = std::move(jobs.front());
+                jobs.pop_front();
+            }
+            const int rc = run_job(j);
+            {
+                std::lock_guard<std::mutex> lk(mu);
+                if (rc != MOE_OK && err == MOE_OK) { err = rc; err_msg = moe_last_error(); }
+                issued = j.seq;
+            }
+            cv_done.notify_all();
+        }
+    }
+    // blocks until the copies of job `seq` have been enqueued on the copy stream
+    int wait_issued(uint64_t seq) {
+        std::unique_lock<std::mutex> lk(mu);
+        cv_done.wait(lk, [&] { return issued >= seq; });
+        if (err != MOE_OK) { moe::set_error("bounce copy worker: %s", err_msg.c_str()); return err; }
+        return MOE_OK;
+    }
+    void shutdown() {
+        if (worker.joinable()) {
+            { std::lock_guard<std::mutex> lk(mu); stop = true; }
+            cv_job.notify_all();
+            worker.join();
+        }
+        for (size_t i = 0; i < chunk.size(); ++i) {
+            if (backend == MOE_STAGE_DEVICE) { if (chunk[i]) (void)hipHostFree(chunk[i]); if (done[i]) (void)hipEventDestroy(done[i]); }
+            else std::free(chunk[i]);
+        }
+        chunk.clear(); done.clear(); busy.clear();
+        n_chunks = 0;
+    }
+};
+
 }  // namespace
 
 struct moe_stager {
     int backend = MOE_STAGE_DEVICE;
+    Bounce bounce;
     hipStream_t copy_stream = nullptr;
     std::vector<Type> types;
     std::vector<Module> modules;
@@ -87,7 +200,28 @@ int copy_into(moe_stager* st, int id, int slot) {
     Module& m = st->modules[id];
     Type& t = st->types[m.type];
     uint8_t* dst = t.mem + (size_t)slot * t.slot_bytes;
-    if (st->backend == MOE_STAGE_DEVICE) {
+    if (m.pageable) {
+        Bounce& b = st->bounce;
+        if (b.n_chunks == 0) {
+            moe::set_error("module %d has pageable sources but no bounce ring is configured (moe_stage_set_bounce)", id);
+            return MOE_ERR_STATE;
+        }
+        BounceJob j;
+        j.dst = dst;
+        j.pieces = m.pieces;
+        j.ready = m.ready;
+        if (st->backend == MOE_STAGE_DEVICE && t.freed_valid[slot]) {
+            j.wait_for = t.freed[slot];
+            t.freed_valid[slot] = 0;
+        }
+        {
+            std::lock_guard<std::mutex> lk(b.mu);
+            j.seq = ++b.enqueued;
+            m.job_seq = j.seq;
+            b.jobs.push_back(std::move(j));
+        }
+        b.cv_job.notify_one();
+    } else if (st->backend == MOE_STAGE_DEVICE) {
         if (t.freed_valid[slot]) {
             MOE_HIP_CHECK(hipStreamWaitEvent(st->copy_stream, t.freed[slot], 0));
             t.freed_valid[slot] = 0;
@@ -126,7 +260,10 @@ int pump_type(moe_stager* st, int ti) {
     const int id = t.fifo.front();
     t.fifo.pop_front();
     int rc = copy_into(st, id, slot);
-    if (rc != MOE_OK) return rc;
+    if (rc != MOE_OK) {
+        t.fifo.push_front(id);   // not copied: it keeps its turn
+        return rc;
+    }
     t.fifo.push_back(id);  // the reference pushes the name back for the next pass
     return 1;
 }
@@ -188,6 +325,10 @@ int drop_residency(moe_stager* st, int ti, const char* who) {
             moe::set_error("%s: module %d of type %d is still held (release it first)", who, t.owner[s], ti);
             return MOE_ERR_STATE;
         }
+    if (st->bounce.n_chunks > 0) {
+        int rc = st->bounce.wait_issued(st->bounce.enqueued);
+        if (rc != MOE_OK) return rc;
+    }
     if (st->backend == MOE_STAGE_DEVICE) MOE_HIP_CHECK(hipStreamSynchronize(st->copy_stream));
     for (int s = 0; s < t.n_total; ++s) {
         if (t.owner[s] >= 0) {
@@ -282,6 +423,59 @@ extern "C" int moe_stage_add_module(moe_stager* st, int32_t type, int32_t n_tens
     return id;
 }
 
+extern "C" int moe_stage_set_bounce(moe_stager* st, int32_t n_chunks, size_t chunk_bytes, int32_t n_threads) {
+    MOE_REQUIRE(st, "moe_stage_set_bounce: NULL stager");
+    MOE_REQUIRE(n_chunks >= 2 && n_chunks <= 256, "moe_stage_set_bounce: n_chunks %d outside [2,256]", n_chunks);
+    MOE_REQUIRE(chunk_bytes >= 4096 && chunk_bytes <= ((size_t)1 << 32), "moe_stage_set_bounce: chunk_bytes %zu outside [4096, 4 GiB]",
+                chunk_bytes);
+    MOE_REQUIRE(n_threads >= 1 && n_threads <= 64, "moe_stage_set_bounce: n_threads %d outside [1,64]", n_threads);
+    std::lock_guard<std::mutex> lk(st->mu);
+    Bounce& b = st->bounce;
+    MOE_REQUIRE(b.n_chunks == 0, "moe_stage_set_bounce: the bounce ring is already configured");
+    b.backend = st->backend;
+    b.stream = st->copy_stream;
+    b.chunk_bytes = chunk_bytes;
+    b.n_threads = n_threads;
+    if (st->backend == MOE_STAGE_DEVICE) MOE_HIP_CHECK(hipGetDevice(&b.device));
+    for (int i = 0; i < n_chunks; ++i) {
+        uint8_t* p = nullptr;
+        hipEvent_t ev = nullptr;
+        if (st->backend == MOE_STAGE_DEVICE) {
+            // pinned memory is ALLOCATED here; existing memory is never registered
+            hipError_t e = hipHostMalloc(reinterpret_cast<void**>(&p), chunk_bytes, hipHostMallocDefault);
+            if (e == hipSuccess) e = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
+            if (e != hipSuccess) {
+                if (p) (void)hipHostFree(p);
+                moe::set_error("moe_stage_set_bounce: chunk %d of %zu bytes: %s", i, chunk_bytes, hipGetErrorString(e));
+                b.shutdown();
+                return MOE_ERR_HIP;
+            }
+        } else {
+            p = static_cast<uint8_t*>(std::malloc(chunk_bytes));
+            if (!p) {
+                moe::set_error("moe_stage_set_bounce: out of memory for chunk %d", i);
+                b.shutdown();
+                return MOE_ERR_INVALID;
+            }
+        }
+        b.chunk.push_back(p);
+        b.done.push_back(ev);
+        b.busy.push_back(0);
+    }
+    b.n_chunks = n_chunks;
+    b.worker = std::thread([&b] { b.loop(); });
+    return MOE_OK;
+}
+
+extern "C" int moe_stage_add_module_pageable(moe_stager* st, int32_t type, int32_t n_tensors, const void* const* src,
+                                             const size_t* bytes, const size_t* dst_offsets) {
+    int id = moe_stage_add_module(st, type, n_tensors, src, bytes, dst_offsets);
+    if (id < 0) return id;
+    std::lock_guard<std::mutex> lk(st->mu);
+    st->modules[id].pageable = true;
+    return id;
+}
+
 extern "C" int moe_stage_pump(moe_stager* st) {
     MOE_REQUIRE(st, "moe_stage_pump: NULL stager");
     std::lock_guard<std::mutex> lk(st->mu);
@@ -305,6 +499,10 @@ extern "C" int moe_stage_acquire(moe_stager* st, int32_t id, void* stream, int32
                            "(release or clear earlier modules first)", id, m.type);
             return MOE_ERR_STATE;
         }
+    }
+    if (m.pageable) {   // the worker must have enqueued this module's copies (and recorded `ready`) before anyone waits on it
+        int rc = st->bounce.wait_issued(m.job_seq);
+        if (rc != MOE_OK) return rc;
     }
     if (st->backend == MOE_STAGE_DEVICE) MOE_HIP_CHECK(hipStreamWaitEvent(moe::as_stream(stream), m.ready, 0));
     m.held = true;
@@ -491,12 +689,17 @@ extern "C" int moe_stage_stats(moe_stager* st, int64_t* n_copies, int64_t* n_byt
 extern "C" int moe_stage_sync(moe_stager* st) {
     MOE_REQUIRE(st, "moe_stage_sync: NULL stager");
     std::lock_guard<std::mutex> lk(st->mu);
+    if (st->bounce.n_chunks > 0) {
+        int rc = st->bounce.wait_issued(st->bounce.enqueued);
+        if (rc != MOE_OK) return rc;
+    }
     if (st->backend == MOE_STAGE_DEVICE) MOE_HIP_CHECK(hipStreamSynchronize(st->copy_stream));
     return MOE_OK;
 }
 
 extern "C" int moe_stage_destroy(moe_stager* st) {
     if (!st) return MOE_OK;
+    st->bounce.shutdown();   // (joins the worker: queued jobs are finished first)
     if (st->backend == MOE_STAGE_DEVICE) {
         (void)hipStreamSynchronize(st->copy_stream);
         for (Module& m : st->modules)

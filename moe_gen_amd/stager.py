@@ -47,7 +47,10 @@ class Stager:
     n_slots: {module_type: slots in the prefill phase}; n_slots_decoding: optional larger
     counts for the decoding phase (num_decoding_module_buffer, :918-927);
     backend "device": slots in HBM, sources must be pinned host tensors;
-    backend "host": slots in host memory, plain memcpy (host-only tests)."""
+    backend "host": slots in host memory, plain memcpy (host-only tests);
+    bounce_chunks > 0: a ring of that many pinned chunks of bounce_chunk_bytes through which modules
+    whose sources lie in ordinary (pageable) memory are copied (Arena.stream_from,
+    add_module(..., pageable=True)), bounce_threads host threads per chunk fill."""
 
     # free_weights_buffer records an event on the caller's stream and the next copy into the slot
     # waits for it: a caller need not drain its stream before letting go of weights (the
@@ -56,7 +59,8 @@ class Stager:
 
     def __init__(self, module_shapes: dict, n_slots: dict, device="cuda", n_slots_decoding: dict | None = None,
                  model_type: str = "", num_hidden_layers: int = 0, num_local_experts: int = 0,
-                 backend: str = "device"):
+                 backend: str = "device", bounce_chunks: int = 0, bounce_chunk_bytes: int = 32 << 20,
+                 bounce_threads: int = 8):
         self.backend = backend
         self.device = torch.device("cpu") if backend == "host" else torch.device(device)
         self.model_type = model_type
@@ -91,6 +95,9 @@ class Stager:
             N.check(N.lib().moe_stage_set_phase_slots(self._h, i, self.n_prefill[t],
                                                       max(self.n_prefill[t], self.n_decoding.get(t, 0))),
                     "moe_stage_set_phase_slots")
+        self.bounce = False
+        if bounce_chunks:
+            self.set_bounce(bounce_chunks, bounce_chunk_bytes, bounce_threads)
         self.ids = {}          # module_key -> id
         self.type_of = {}      # module_key -> type
         self._src = []         # keeps the host tensors alive
@@ -99,9 +106,15 @@ class Stager:
     def _stream(self):
         return None if self.backend == "host" else torch.cuda.current_stream().cuda_stream
 
-    def add_module(self, module_key: str, module_type: str, tensors: dict) -> int:
+    def set_bounce(self, n_chunks: int = 8, chunk_bytes: int = 32 << 20, n_threads: int = 8) -> None:
+        """Allocate the ring of pinned chunks that modules with pageable sources travel through."""
+        N.check(N.lib().moe_stage_set_bounce(self._h, n_chunks, chunk_bytes, n_threads), "moe_stage_set_bounce")
+        self.bounce = True
+
+    def add_module(self, module_key: str, module_type: str, tensors: dict, pageable: bool = False) -> int:
         """Register one module (Weights_Storage's module_key -> tensor_key -> host buffer map,
-        core/Weights_Storage/Weights_Storage.cpp:52-90) at the tail of its type's copy queue."""
+        core/Weights_Storage/Weights_Storage.cpp:52-90) at the tail of its type's copy queue.
+        pageable: the tensors lie in ordinary host memory and go through the bounce ring."""
         lay = self.layout[module_type]
         if set(tensors) != set(lay):
             raise RuntimeError(f"module {module_key}: tensors {sorted(tensors)} do not match the slot layout {sorted(lay)}")
@@ -111,12 +124,16 @@ class Stager:
             t = tensors[name]
             if tuple(t.shape) != shape or t.dtype != dtype or not t.is_contiguous() or t.is_cuda:
                 raise RuntimeError(f"module {module_key}.{name}: expected a contiguous host {dtype} tensor of shape {shape}")
-            if self.backend == "device" and not t.is_pinned():
-                raise RuntimeError(f"module {module_key}.{name}: host tensor must be pinned (allocate with pin_memory=True)")
+            if self.backend == "device" and not pageable and not t.is_pinned():
+                raise RuntimeError(f"module {module_key}.{name}: host tensor must be pinned (allocate with pin_memory=True), "
+                                   "or registered with pageable=True on a stager with a bounce ring")
             src.append(t.data_ptr()); nbytes.append(b); offs.append(off)
             self._src.append(t)
-        mid = N.lib().moe_stage_add_module(self._h, self.types.index(module_type), n, (ctypes.c_void_p * n)(*src),
-                                           (ctypes.c_size_t * n)(*nbytes), (ctypes.c_size_t * n)(*offs))
+        if pageable and not self.bounce:
+            self.set_bounce()
+        add = N.lib().moe_stage_add_module_pageable if pageable else N.lib().moe_stage_add_module
+        mid = add(self._h, self.types.index(module_type), n, (ctypes.c_void_p * n)(*src),
+                  (ctypes.c_size_t * n)(*nbytes), (ctypes.c_size_t * n)(*offs))
         if mid < 0:
             N.check(mid, "moe_stage_add_module")
         self._register(module_key, module_type, mid)
@@ -143,14 +160,18 @@ class Stager:
             if entries[name][1] != b or tuple(entries[name][2]) != shape:
                 raise RuntimeError(f"module {module_key}.{name}: arena entry {entries[name][1:]} does not match "
                                    f"the slot layout ({b} bytes, shape {shape})")
-        if self.backend == "device" and not arena.data.is_pinned():
-            raise RuntimeError("the arena must be pinned host memory (allocate it with pin_memory=True)")
+        pageable = bool(getattr(arena, "pageable", False))
+        if self.backend == "device" and not pageable and not arena.data.is_pinned():
+            raise RuntimeError("the arena must be pinned host memory (allocate it with pin_memory=True), or a "
+                               "segment adopted with Arena.stream_from")
+        if pageable and not self.bounce:
+            self.set_bounce()
         n = len(lay)
         keys = (ctypes.c_char_p * n)(*[k.encode() for k in lay])
         offs = (ctypes.c_size_t * n)(*[v[0] for v in lay.values()])
-        mid = N.lib().moe_stage_add_module_from_arena(self._h, self.types.index(module_type), arena.index._h,
-                                                      module_key.encode(), arena.data.data_ptr(), arena.data.numel(),
-                                                      n, keys, offs)
+        add = N.lib().moe_stage_add_module_from_segment if pageable else N.lib().moe_stage_add_module_from_arena
+        mid = add(self._h, self.types.index(module_type), arena.index._h, module_key.encode(), arena.data.data_ptr(),
+                  arena.data.numel(), n, keys, offs)
         if mid < 0:
             N.check(mid, "moe_stage_add_module_from_arena")
         self._src.append(arena)

@@ -317,3 +317,39 @@ def test_arena_to_hbm():
                 assert torch.equal(w[n].view(torch.uint8).cpu(), t.view(torch.uint8)), (mk, n)
             st.free_weights_buffer(mk)
     st.close()
+
+
+@pytest.mark.parametrize("chunk_bytes", [1 << 16, 1 << 22])
+def test_segment_to_hbm_through_the_bounce_ring(chunk_bytes):
+    """Modules registered from a weight segment in ORDINARY host memory (Arena.stream_from: nothing is copied into
+    pinned memory up front) arrive in their HBM slots byte for byte through the stager's ring of pinned chunks --
+    pieces smaller than a chunk and pieces of many chunks, more modules than slots, three passes -- while the
+    consumer's stream only ever waits on events."""
+    from moe_gen_amd import Arena, Stager
+    shapes = {"routed_expert": {"gate_proj.weight": ((256, 1024), torch.float8_e4m3fn),      # 256 KiB
+                                "up_proj.weight": ((256, 1024), torch.float8_e4m3fn),
+                                "down_proj.weight": ((1024, 2560), torch.float8_e4m3fn),     # 2.5 MiB
+                                "tiny": ((3, 5), torch.float32)}}
+    print(f"bounce ring, chunks of {chunk_bytes} bytes", flush=True)
+    g = torch.Generator().manual_seed(2)
+    mods = {f"routed_expert_{L}_{e}": {n: (torch.randint(0, 255, s, generator=g, dtype=torch.uint8).view(d) if d != torch.float32
+                                           else torch.randn(s, generator=g))
+                                       for n, (s, d) in shapes["routed_expert"].items()} for L in (2, 3, 4) for e in range(6)}
+    packed = Arena.pack(mods, pin=False)
+    arena = Arena.stream_from(packed.index.serialize(), packed.data)
+    assert arena.pageable and not arena.data.is_pinned()
+    st = Stager(shapes, {"routed_expert": 4}, model_type="deepseek_v3", num_hidden_layers=5, num_local_experts=6,
+                bounce_chunks=4, bounce_chunk_bytes=chunk_bytes, bounce_threads=4)
+    for mk in mods:
+        st.add_module_from_arena(mk, "routed_expert", arena)
+    for rep in range(3):
+        for mk, tensors in mods.items():
+            w = st.get_weights(mk)
+            got = {n: t.clone() for n, t in w.items()}          # on the current stream, behind the hand-off event
+            st.free_weights_buffer(mk)
+            torch.cuda.synchronize()
+            for n, t in tensors.items():
+                assert torch.equal(got[n].view(torch.uint8).cpu(), t.view(torch.uint8)), (rep, mk, n)
+    copies, nbytes = st.stats()
+    assert copies >= 3 * len(mods)
+    st.close()

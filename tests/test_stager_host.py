@@ -276,3 +276,70 @@ def test_pool_size_in_the_decoding_phase_follows_the_pool():
     assert st2.pool_size("routed_expert") == 2
     st2.set_phase("decoding")
     assert st2.pool_size("routed_expert") == 6 and st2.pool_size("shared_expert") == 1
+
+
+@pytest.mark.parametrize("chunk_bytes,threads", [(4096, 1), (8192, 3), (1 << 22, 4)])
+def test_pageable_segment_through_the_bounce_ring(chunk_bytes, threads):
+    """A weight segment adopted where it lies, in ordinary host memory (Arena.stream_from: the reference maps its
+    shm segment once and views it, Weights_Storage.cpp:52-78), reaches the slots through the stager's ring of
+    bounce chunks byte for byte: pieces smaller than, equal to and several times a chunk, more modules than slots,
+    several passes (chunks and slots are reused), skipped modules reclaimed by clear_expert_buffer, and a reset in
+    between.  Host backend: the chunks are plain memory and the transfer out of a chunk is a memcpy."""
+    from moe_gen_amd import Arena
+    shapes = {"routed_expert": {"gate_proj.weight": ((96, 128), torch.bfloat16),        # 24576 bytes
+                                "up_proj.weight": ((32, 128), torch.bfloat16),          # 8192
+                                "down_proj.weight": ((1300, 1024), torch.float32)}}     # 5.3 MB: above 1 MiB per thread
+    E, L, slots = 5, 3, 3        # (three layers: with two, the layer before the current one is also the next one, and
+    g = torch.Generator().manual_seed(5)   #  the rule that drops the previous layer's leftovers drops what was just prefetched)
+    mods = {f"routed_expert_{lay}_{e}": {n: torch.randn(s, generator=g).to(d) for n, (s, d) in shapes["routed_expert"].items()}
+            for lay in range(L) for e in range(E)}
+    packed = Arena.pack(mods, pin=False)
+    assert not packed.data.is_pinned()
+    arena = Arena.stream_from(packed.index.serialize(), packed.data)        # what a process that maps the segment does
+    assert arena.pageable and arena.data.data_ptr() == packed.data.data_ptr()   # adopted in place, not copied
+    st = Stager(shapes, {"routed_expert": slots}, backend="host", model_type="mixtral", num_hidden_layers=L,
+                num_local_experts=E, bounce_chunks=3, bounce_chunk_bytes=chunk_bytes, bounce_threads=threads)
+    for mk in mods:
+        st.add_module_from_arena(mk, "routed_expert", arena)
+    for rounds in range(3):
+        for lay in range(L):
+            for e in range(E):
+                st.clear_expert_buffer(lay, e)
+                if (e + rounds) % 4 == 3:
+                    continue                              # skipped: its slot is reclaimed by a later clear
+                key = f"routed_expert_{lay}_{e}"
+                w = st.get_weights(key)
+                for n, t in mods[key].items():
+                    assert torch.equal(w[n], t), (rounds, key, n)
+                st.free_weights_buffer(key)
+        if rounds == 1:
+            st.reset_prefill_buffer(); st.reset_weight_copy_queue()      # drains the worker's queue first
+    st.sync()
+    copies, nbytes = st.stats()
+    per_module = sum(t.numel() * t.element_size() for t in mods["routed_expert_0_0"].values())
+    assert copies >= 3 * L * (E - 2) and nbytes == copies * per_module
+    st.close()
+
+
+def test_pageable_module_without_a_bounce_ring_is_an_error():
+    """Through the C ABI alone: a module registered as pageable cannot be copied before moe_stage_set_bounce."""
+    import ctypes
+    from moe_gen_amd import _native as N
+    L = N.lib()
+    nb = 256
+    pool = (ctypes.c_uint8 * (2 * nb))()
+    h = ctypes.c_void_p()
+    N.check(L.moe_stage_create(ctypes.byref(h), 1, (ctypes.c_size_t * 1)(nb), (ctypes.c_int32 * 1)(2),
+                               (ctypes.c_void_p * 1)(ctypes.addressof(pool)), 1), "create")
+    src = (ctypes.c_uint8 * nb)(*range(nb))
+    mid = L.moe_stage_add_module_pageable(h, 0, 1, (ctypes.c_void_p * 1)(ctypes.addressof(src)), (ctypes.c_size_t * 1)(nb),
+                                          (ctypes.c_size_t * 1)(0))
+    assert mid == 0
+    slot = ctypes.c_int32(-1)
+    assert L.moe_stage_acquire(h, mid, None, ctypes.byref(slot)) != 0 and "bounce" in N.last_error()
+    assert L.moe_stage_set_bounce(h, 1, 4096, 1) == -1 and "n_chunks" in N.last_error()
+    N.check(L.moe_stage_set_bounce(h, 2, 4096, 2), "set_bounce")
+    assert L.moe_stage_set_bounce(h, 2, 4096, 2) == -1 and "already" in N.last_error()
+    N.check(L.moe_stage_acquire(h, mid, None, ctypes.byref(slot)), "acquire")
+    assert bytes(pool[slot.value * nb:(slot.value + 1) * nb]) == bytes(src)
+    L.moe_stage_destroy(h)
