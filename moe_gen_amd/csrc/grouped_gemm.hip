@@ -56,6 +56,7 @@ constexpr int BK = 64;           // k per stage (bf16 elements); 128 bytes per L
 constexpr int ROW_B = 128;       // bytes per LDS row
 constexpr int BN_ROWS = 256;     // weight rows per workgroup (128 gate + 128 up when SWIGLU)
 constexpr int MAX_E = 1024;
+constexpr int PAIR_LO = 257, PAIR_HI = 384;   // bf16: rows of an expert that runs as two tiles of the 192-row body
 
 __device__ __forceinline__ float bf16r(float a) { return __uint_as_float(pack_bf16(a, 0.0f) << 16); }
 
@@ -89,6 +90,7 @@ struct GemmArgs {
     int rem_split;              // 1: the rule applies to what an expert's full 256-row tiles leave over (count % 256)
                                 // instead of to its count: the persistent kernel takes the full tiles, and the
                                 // last, ragged one only if it holds more than cold_max rows
+    int pair_rows;              // 1: experts of PAIR_LO .. PAIR_HI rows also belong to the one-workgroup-per-tile kernel
     int tail_cus;               // > 0: the persistent kernel runs whole rounds of this many tiles (one per CU); what
                                 // is left, if at most half a round, goes to the other kernel as 128-row half tiles
 };
@@ -814,9 +816,13 @@ __device__ __forceinline__ void stream8_tile(const GemmArgs& g, uint8_t* buf0, u
 // 192-row body does not fit the registers) run side by side on one XCD and take the weights with plain loads, so
 // that all but the first read of a line come out of that XCD's L2.
 // 256-row tiles of an expert with `count` rows in the persistent kernel's tile space
+// whether an expert of `count` rows belongs to the one-workgroup-per-tile kernel (no rem_split)
+__device__ __forceinline__ bool is_cold(const GemmArgs& g, int count) {
+    return count <= g.cold_max || (g.pair_rows && count >= PAIR_LO && count <= PAIR_HI);
+}
 __device__ __forceinline__ int persistent_tiles(const GemmArgs& g, int count) {
     if (g.rem_split) return (count >> 8) + ((count & 255) > g.cold_max ? 1 : 0);
-    return count <= g.cold_max ? 0 : (count + 255) >> 8;
+    return is_cold(g, count) ? 0 : (count + 255) >> 8;
 }
 // How many tiles at the end of that space the persistent kernel leaves to the other kernel.  One workgroup per CU
 // walks the space in rounds of tail_cus tiles, and a last round of a few tiles costs as much as a full one while
@@ -829,7 +835,19 @@ __device__ __forceinline__ int tail_tiles(const GemmArgs& g, int total) {
 }
 
 template <int SINGLE>   // rows that one tile may hold
-__device__ __forceinline__ int tiles_of(int count) { return count <= SINGLE ? (count > 0 ? 1 : 0) : (count + 127) >> 7; }
+__device__ __forceinline__ int tiles_of(int count) {
+    if (count <= SINGLE) return count > 0 ? 1 : 0;
+    // bf16 weights: an expert of 257 to 384 rows is cut in the middle, into two tiles of the 192-row body that run
+    // side by side on one XCD and share the weights through its L2: 320 rows are 2 x 160 rows of MFMA work, where
+    // two 256-row tiles of the persistent kernel multiply 512 and three 128-row tiles read the weights three times.
+    // Mixtral-8x22B shapes, 8 experts of 288 / 320 / 384 rows: gate/up 1.31 / 1.29 / 1.30 -> 1.07 / 1.13 / 1.17 ms,
+    // down projection within 4 % either way; up to 256 rows one tile of the persistent kernel stays better (224
+    // rows: 0.82 against 1.01 ms).
+    if (SINGLE == 192 && count > PAIR_LO - 1 && count <= PAIR_HI) return 2;
+    return (count + 127) >> 7;
+}
+// rows of either tile of such a pair (the first tile holds whole 16-row groups)
+__device__ __forceinline__ int half_rows(int count) { return ((count + 1) / 2 + 15) & ~15; }
 
 // One workgroup per (M tile, N tile); serves what the persistent kernel does not take (few rows per expert, odd K).
 template <int WN, bool SWIGLU, bool W8>
@@ -850,7 +868,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     const bool s8_ok = !g.row_map || g.a_bytes < (1ull << 32);   // (the weight streamer addresses gathered rows with 32-bit offsets)
     int run = mtile_prefix_scan<NT>(g, tid, s_pref, s_wtot, mine, [&](int c) {
         if (g.rem_split) c &= 255;      // the rows the persistent kernel's full tiles leave over
-        return c > g.cold_max ? 0 : tiles_of<(W8 ? 128 : 192)>(c);
+        return (g.rem_split ? c > g.cold_max : !is_cold(g, c)) ? 0 : tiles_of<(W8 ? 128 : 192)>(c);
     }, [](int, int, int) {});
     const int total = run * g.n_tiles_n;
 
@@ -924,7 +942,10 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     if (row_end - first_row <= 64) gemm_tile<1, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
     else if (row_end - first_row <= 128) gemm_tile<2, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
     else if (!W8 && mt_e == 1) gemm_tile<3, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
-    else gemm_tile<2, WN, SWIGLU, W8, false>(g, smem0, smem1, e, first_row + m_tile * 128, row_end, n_tile);
+    else if (!W8 && row_end - first_row >= PAIR_LO && row_end - first_row <= PAIR_HI) {
+        const int r0 = first_row + m_tile * half_rows(row_end - first_row);
+        gemm_tile<3, WN, SWIGLU, W8, false>(g, smem0, smem1, e, r0, min(row_end, r0 + half_rows(row_end - first_row)), n_tile);
+    } else gemm_tile<2, WN, SWIGLU, W8, false>(g, smem0, smem1, e, first_row + m_tile * 128, row_end, n_tile);
 }
 
 // lane id produced where it is used: the compiler cannot hoist it (and everything derived from it)
@@ -1254,7 +1275,7 @@ template <int WN, bool SWIGLU, bool W8>
 int launch_tiles(const GemmArgs& g, int n_rows, hipStream_t st) {
     auto kern = grouped_gemm_kernel<WN, SWIGLU, W8>;
     // sum_e tiles_of(c_e) <= sum_e (c_e / 128 + 1); with the larger experts elsewhere, one tile per expert that has rows
-    const long max_mtiles = g.cold_max <= 192 ? (g.E < n_rows ? g.E : n_rows) : (long)n_rows / 128 + g.E;
+    const long max_mtiles = g.cold_max <= 192 ? (g.pair_rows ? 2 : 1) * (long)(g.E < n_rows ? g.E : n_rows) : (long)n_rows / 128 + g.E;
     // (+ the persistent kernel's last tiles, at most half a round of them, as two half tiles each)
     const long grid = ((max_mtiles * g.n_tiles_n + g.tail_cus + 31) / 32) * 32;   // whole rounds of 8 groups of 4 tiles
     if (grid > 0x7fffffffL) {
@@ -1320,6 +1341,7 @@ int launch_mt(const GemmArgs& g0, int n_rows, hipStream_t st) {
     // for the persistent kernel's last round anyway.)
     g.cold_max = W8 ? 128 : 192;
     g.rem_split = W8 ? 1 : 0;
+    g.pair_rows = W8 ? 0 : 1;
     // Last round of the persistent kernel (tail_tiles above): Mixtral-8x22B, 8192 tokens, down projection (6.4 rounds
     // of 0.4 ms) 2.82 -> 2.66 ms, step 8.31 -> 8.13; Mixtral-8x7B 9.39 -> 9.27 ms; DeepSeek-V2-Lite 0.855 -> 0.821 ms
     // (its shared expert's 128 down tiles become 256 half tiles: 0.071 -> 0.055 ms); DeepSeek-V2-236B 11.43 -> 11.46,
