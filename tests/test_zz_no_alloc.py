@@ -58,6 +58,44 @@ def test_static_dispatch_matches_dispatch_on_consecutive_calls():
     assert got[0].sum().item() == 0 and got[1].sum().item() == 0
 
 
+@pytest.mark.gpu
+def test_static_dispatch_captured_in_a_graph():
+    """The use the entry point is documented for: after one eager call on the device (which looks the array's
+    address up), further calls are captured into a HIP graph -- three kernel launches, no allocation, no memset --
+    and every replay, with the program's own eager work and synchronisations in between and with new routing in the
+    same buffers, gives what moe_dispatch gives eagerly."""
+    n, k, E = 5000, 6, 160
+    print(f"no-alloc dispatch under graph capture: {n}x{k}/{E}", flush=True)
+    L = N.lib()
+    idx_static = _idx(n, k, E, 11)
+    _run("moe_dispatch_static", idx_static, E)                       # eager: resolves the symbol address on this device
+    i32 = dict(dtype=torch.int32, device="cuda")
+    counts, offsets = torch.zeros(E, **i32), torch.zeros(E + 1, **i32)
+    perm, pos, row_map = (torch.zeros(n * k, **i32) for _ in range(3))
+    p = lambda t: t.data_ptr()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                                    # warm-up on the side stream, as torch asks before a capture
+        N.check(L.moe_dispatch_static(p(idx_static), n, k, E, p(counts), p(offsets), p(perm), p(pos), p(row_map), None, 0, None,
+                                      side.cuda_stream), "moe_dispatch_static")
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = L.moe_dispatch_static(p(idx_static), n, k, E, p(counts), p(offsets), p(perm), p(pos), p(row_map), None, 0, None,
+                                   torch.cuda.current_stream().cuda_stream)
+    N.check(rc, "moe_dispatch_static under capture")
+    torch.cuda.synchronize()
+    for it in range(4):
+        idx_static.copy_(_idx(n, k, E, 20 + it))                     # new routing in the captured buffers
+        for t in (counts, offsets, perm, pos, row_map):
+            t.fill_(-3)
+        graph.replay()
+        torch.cuda.synchronize()
+        want = _run("moe_dispatch", idx_static, E)                    # eager work of the program between the replays
+        for name, a, b in zip(("counts", "offsets", "perm", "pos", "row_map"), want, (counts, offsets, perm, pos, row_map)):
+            assert torch.equal(a, b), (it, name)
+
+
 def test_static_dispatch_rejects_what_does_not_fit():
     """Size and argument checks happen on the host, before anything touches a device."""
     L = N.lib()
