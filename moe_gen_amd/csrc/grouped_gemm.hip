@@ -636,13 +636,15 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
 //    request, 128 k at a time, into the wave's own 4 KiB of a buffer: no staging registers, no LDS stores, half the
 //    bytes, and three buffers keep two 128-k blocks in flight per CU;
 //  * a lane reads 16 consecutive fp8 weights of its fragment row (one ds_read_b128), which after conversion are its
-//    A operands of BOTH 32-wide k-steps of a 64-k half: lane group q holds k = 16 q + 8 s + (0..7) in step s, and the
-//    token operand reads the chunk that holds those k.  A dot product does not care in which order k is walked,
+//    A operands of BOTH 32-wide k-steps of a 64-k half: lane group q holds k = 16 f(q) + 8 s + (0..7) in step s
+//    (f = 0, 2, 1, 3), and the token operand reads the chunk that holds those k.  A dot product does not care in which order k is walked,
 //    and the order depends on nothing but the column: a row's result does not depend on its tile or its neighbours.
 // LDS layouts (the DMA lets every lane fetch what belongs at its place, so swizzles are free):
 //  weights: 128-byte rows, 16-byte part c of fragment row r at part c ^ wsw(r); tokens: 256-byte rows (128 k), chunk
 //  c of row r at chunk c ^ tsw(r).  The LDS serves lanes 8 i .. 8 i + 7 together with lanes 32 + 8 i .. (the same 8
-//  rows, lane groups q and q + 2): with these keys their 16 reads fall on 16 different bank groups.
+//  rows, lane groups q and q + 2, whose chunks f(q) and f(q + 2) = f(q) + 1 are neighbours): with these keys their 16
+//  reads fall on 16 different bank groups.  (Measured with 8 waves reading back to back: 32 cycles per wave and
+//  ds_read_b128 for both layouts, 55 with lane group q on chunk q.)
 __device__ __forceinline__ int wsw(int r) { return ((r >> 1) & 1) | (((r >> 2) & 1) << 2); }
 __device__ __forceinline__ int tsw(int r) { return (r & 3) | ((r & 4) << 1); }
 
@@ -689,17 +691,19 @@ __device__ __forceinline__ void stream8_tile(const GemmArgs& g, uint8_t* buf0, u
         w_voff[i] = (uint32_t)min(n0 + rt, N - 1) * (uint32_t)K + (uint32_t)((pp ^ wsw(fr)) << 4);
     }
     // tokens, instruction i: rows 8 wave + 4 i + lane / 16 of the 64 staged, chunk lane % 16.  Gathered rows go through
-    // one descriptor over x (a row_map entry outside x reads zeros), sorted rows through one that starts at the tile.
+    // one descriptor over x (a row_map entry outside x reads zeros), sorted rows through one that holds the tile's rows
+    // and nothing else.  Rows past the expert's last get an offset past either descriptor: zeros arrive in LDS
+    // without a request to memory (nobody uses the products of those rows; the instruction still counts).
     uint32_t t_voff[NDT];
     const uint8_t* a_base = reinterpret_cast<const uint8_t*>(g.a) + (g.row_map ? (size_t)0 : (size_t)row0 * K * 2);
-    const int a_records = g.row_map ? (int)(uint32_t)g.a_bytes : -1;
+    const int a_records = g.row_map ? (int)(uint32_t)g.a_bytes : (row_end - row0) * K * 2;
 #pragma unroll
     for (int i = 0; i < NDT; ++i) {
         const int tr = 8 * wave + 4 * i + (lane >> 4);
         const int r = min(row0 + tr, row_end - 1);
         const int src = g.row_map ? ((gptr_i32)(uintptr_t)g.row_map)[r] : r - row0;
         t_voff[i] = (uint32_t)src * (uint32_t)(K * 2) + (uint32_t)(((lane & 15) ^ tsw(tr)) << 4);
-        if (g.row_map && (unsigned)src >= (unsigned)g.a_rows) t_voff[i] = 0xfffffff0u;      // past any descriptor: zeros
+        if (row0 + tr >= row_end || (g.row_map && (unsigned)src >= (unsigned)g.a_rows)) t_voff[i] = 0xfffffff0u;
     }
     float rsc[2][2];                              // block scales of the block being multiplied / of the next one
     auto scales = [&](int p_pipe, int set) {
@@ -711,25 +715,30 @@ __device__ __forceinline__ void stream8_tile(const GemmArgs& g, uint8_t* buf0, u
             rsc[set][j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, 0, (srow[j] + pr) * 4, 0));
         }
     };
-    auto dma = [&](int p_pipe, uint8_t* buf) {
+    // DMA instruction i of a block: 0 .. NDW-1 weights (read once: non-temporal, which is worth 5 % of the stream),
+    // NDW .. NDW+NDT-1 tokens
+    auto dma_one = [&](int p_pipe, uint8_t* buf, int i) __attribute__((always_inline)) {
         // past the end of k nobody reads what arrives: an empty descriptor returns zeros without touching memory,
         // and the instruction still counts
         const int live = uni(p_pipe < npair ? -1 : 0);   // (a scalar, or the descriptor ends up in vector registers)
         int pr = min(p_pipe, npair - 1) + prot;
         pr = pr >= npair ? pr - npair : pr;
-#pragma unroll
-        for (int i = 0; i < NDW; ++i) {
+        if (i < NDW) {
             const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)bmat[i >> 1], 0, live, 0x00020000);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_u8)(buf + wave * 4096 + i * 1024), 16, w_voff[i], (uint32_t)(pr * 128), 0, 0);
-        }
-        const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)a_base, 0, live & a_records, 0x00020000);
-#pragma unroll
-        for (int i = 0; i < NDT; ++i)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_u8)(buf + S8_WBYTES + wave * 2048 + i * 1024), 16, t_voff[i],
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_u8)(buf + wave * 4096 + i * 1024), 16, w_voff[i], (uint32_t)(pr * 128), 0, 2);
+        } else {
+            const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)a_base, 0, live & a_records, 0x00020000);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_u8)(buf + S8_WBYTES + wave * 2048 + (i - NDW) * 1024), 16, t_voff[i - NDW],
                                                      (uint32_t)(pr * 256), 0, 0);
+        }
+    };
+    auto dma = [&](int p_pipe, uint8_t* buf) {
+#pragma unroll
+        for (int i = 0; i < NDW + NDT; ++i) dma_one(p_pipe, buf, i);
     };
 
     const int frow = lane & 15, q = lane >> 4;
+    const int fq = ((q & 1) << 1) | (q >> 1);
     const uint32_t w_rd = (uint32_t)(wave * 4096 + frow * 128), wkey = (uint32_t)wsw(frow);
     const uint32_t t_rd = (uint32_t)(S8_WBYTES + frow * 256), tkey = (uint32_t)tsw(frow);   // (group bases are multiples of 16)
     f32x4 acc[TG][2];
@@ -739,8 +748,8 @@ __device__ __forceinline__ void stream8_tile(const GemmArgs& g, uint8_t* buf0, u
     // Iteration p multiplies block p out of buffer p % 3.  Before it: this wave's DMA of block p has landed (at most the
     // DMA of block p + 1 is outstanding) and its LDS reads have returned, then everybody's (a bare s_barrier: a fence
     // would make the compiler wait for ALL outstanding DMA).  After the barrier every wave has left block p - 1,
-    // whose buffer takes block p + 2.  The scale loads come BEFORE the DMA: the compiler's own wait for a scale
-    // counts everything issued after it as allowed to be in flight.
+    // whose buffer takes block p + 2 (its DMA is spread over the iteration).  The scale loads come BEFORE the DMA: the
+    // compiler's own wait for a scale counts everything issued after it as allowed to be in flight.
     auto iteration = [&](int p, const uint8_t* rd, uint8_t* refill, int sset) __attribute__((always_inline)) {
         // (lgkmcnt: this wave's LDS reads of block p - 1 have returned -- its last matrix instructions may be scheduled
         // behind the barrier, and the buffer they read is refilled right after it)
@@ -748,26 +757,33 @@ __device__ __forceinline__ void stream8_tile(const GemmArgs& g, uint8_t* buf0, u
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         scales(p + 1, sset ^ 1);
-        dma(p + 2, refill);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             bf16x8 wa[2][2];
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const u32x4 raw = *reinterpret_cast<const u32x4*>(rd + w_rd + j * 2048 + (((4 * h + q) ^ wkey) << 4));
+                const u32x4 raw = *reinterpret_cast<const u32x4*>(rd + w_rd + j * 2048 + (((4 * h + fq) ^ wkey) << 4));
                 wa[j][0] = __builtin_bit_cast(bf16x8, dequant8(raw[0], raw[1], rsc[sset][j]));
                 wa[j][1] = __builtin_bit_cast(bf16x8, dequant8(raw[2], raw[3], rsc[sset][j]));
             }
 #pragma unroll
             for (int s2 = 0; s2 < 2; ++s2) {
-                const uint32_t coff = (uint32_t)(((8 * h + 2 * q + s2) ^ tkey) << 4);
+                const uint32_t coff = (uint32_t)(((8 * h + 2 * fq + s2) ^ tkey) << 4);
 #pragma unroll
                 for (int t = 0; t < TG; ++t) {
                     const bf16x8 tf = *reinterpret_cast<const bf16x8*>(rd + t_rd + t * 16 * 256 + coff);
                     acc[t][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[0][s2], tf, acc[t][0], 0, 0, 0);
                     acc[t][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[1][s2], tf, acc[t][1], 0, 0, 0);
                 }
+                // the refill of the freed buffer goes out between the four groups of matrix instructions (2, 2, 1, 1
+                // DMA instructions): a wave that issues all six first stands in the memory pipeline's queue while its
+                // matrix instructions wait behind them (3 % at 40-64 rows)
+                const int st = 2 * h + s2;
+                __builtin_amdgcn_sched_barrier(0);
+                dma_one(p + 2, refill, st < 2 ? 2 * st : st + 2);
+                if (st < 2) dma_one(p + 2, refill, 2 * st + 1);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
     };
