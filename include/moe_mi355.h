@@ -198,6 +198,17 @@ int moe_grouped_swiglu_w8a16(const void* x, int32_t x_rows, const int32_t* row_m
                              size_t workspace_bytes, void* stream);
 
 /*
+ * Write n 64-bit words (device pointers of a wave of experts, say) into device memory at dst, from host memory
+ * that may be reused as soon as the call returns: the words travel inside kernel arguments, 256 per launch, on
+ * `stream`, not through the copy engine.  For the per-expert pointer arrays of the two entry points above when
+ * the experts' addresses change from call to call (Expert_Wrapper.get_weights hands out a pool slot per call,
+ * Wrapper.py:496-500, deepseekv3_initializer.py:1259-1266): the table needs no pinned staging buffer whose reuse
+ * would have to wait for a copy, and it does not queue on the copy engine behind the weight copies that the
+ * stager keeps in flight there.  Allocates nothing.
+ */
+int moe_write_words(void* dst, const uint64_t* words, int32_t n, void* stream);
+
+/*
  * Stand-alone block dequantisation (Wrapper.py:109-138), used by tests and by
  * callers that want a bf16 copy:  out = bf16(f32(q) * scale[i/128, j/128]).
  *   q device fp8 [rows, cols]; scale device fp32 [ceil(rows/128), ceil(cols/128)];
@@ -331,7 +342,13 @@ int moe_stage_pump(moe_stager* s);
  * its slot index.  If the module is not yet scheduled, pumps until it is; fails
  * with MOE_ERR_STATE if no slot can become free (all slots held). */
 int moe_stage_acquire(moe_stager* s, int32_t id, void* stream, int32_t* slot);
-/* free_weights_buffer: the slot may be overwritten once `stream` reaches this point. */
+/* free_weights_buffer: the slot may be overwritten once `stream` has finished what it was given before this call.
+ * The event that says so is recorded on `stream` by the next call that copies into a released slot, one event for
+ * all slots released on that stream since the last such call (so `stream` must still exist then); a copy enqueued
+ * behind a wait that is still pending costs the copy stream about 0.2 ms, and ten experts released and refilled
+ * one by one paid it ten times.  The release that leaves the caller holding no module refills the freed slots at
+ * once (the reference's worker refills a slot as soon as it is free, HtoD_Engine.cpp:201-268); while other modules
+ * stay held the refill happens at the next moe_stage_acquire / moe_stage_fetch / moe_stage_pump. */
 int moe_stage_release(moe_stager* s, int32_t id, void* stream);
 /* Copy policy of a module type.  MOE_STAGE_ON_DEMAND turns the cyclic prefetch of that type
  * off: the reference copies every expert of every layer whether or not a token was routed to

@@ -71,6 +71,7 @@ SIGNATURES = {
     "moe_stage_add_module_from_segment": (ctypes.c_int, [c_void_p, c_int32, c_void_p, ctypes.c_char_p, c_void_p, c_size_t,
                                                          c_int32, ctypes.POINTER(ctypes.c_char_p),
                                                          ctypes.POINTER(c_size_t)]),
+    "moe_write_words": (ctypes.c_int, [c_void_p, ctypes.POINTER(ctypes.c_uint64), c_int32, c_void_p]),
     "moe_stage_set_bounce": (ctypes.c_int, [c_void_p, c_int32, c_size_t, c_int32]),
     "moe_stage_add_module_pageable": (ctypes.c_int, [c_void_p, c_int32, c_int32, ctypes.POINTER(c_void_p),
                                                      ctypes.POINTER(c_size_t), ctypes.POINTER(c_size_t)]),

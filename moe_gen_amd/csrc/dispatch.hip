@@ -302,3 +302,29 @@ extern "C" int moe_dispatch_static(const int32_t* topk_idx, int32_t n_tokens, in
     if (rc != MOE_OK) return rc;
     return dispatch_launch(topk_idx, nk, top_k, n_experts, counts, offsets, perm, pos, row_map, x, hidden, xs, seg, st);
 }
+
+// ---- 64-bit words from the host into device memory inside kernel arguments ----
+namespace moe {
+namespace {
+struct WordBlock { uint64_t v[256]; };
+__global__ __launch_bounds__(256) void write_words_kernel(uint64_t* __restrict__ dst, WordBlock w, int n) {
+    const int i = threadIdx.x;
+    if (i < n) dst[i] = w.v[i];
+}
+}  // namespace
+}  // namespace moe
+
+extern "C" int moe_write_words(void* dst, const uint64_t* words, int32_t n, void* stream) {
+    MOE_REQUIRE(n >= 0, "moe_write_words: n %d < 0", n);
+    if (n == 0) return MOE_OK;
+    MOE_REQUIRE(dst && words, "moe_write_words: NULL argument");
+    MOE_REQUIRE((reinterpret_cast<uintptr_t>(dst) & 7) == 0, "moe_write_words: dst is not 8-byte aligned");
+    for (int32_t at = 0; at < n; at += 256) {
+        moe::WordBlock w;
+        const int m = n - at < 256 ? n - at : 256;
+        for (int i = 0; i < m; ++i) w.v[i] = words[at + i];
+        hipLaunchKernelGGL(moe::write_words_kernel, dim3(1), dim3(256), 0, moe::as_stream(stream), static_cast<uint64_t*>(dst) + at, w, m);
+        MOE_HIP_CHECK(hipGetLastError());
+    }
+    return MOE_OK;
+}

@@ -58,7 +58,14 @@ struct Type {
     int n_total = 0, n_active = 0;
     uint8_t* mem = nullptr;
     std::vector<int> owner;             // slot -> module id, -1 free
-    std::vector<hipEvent_t> freed;      // recorded on the consumer stream at release
+    // Hand-back of a slot (device backend).  A release only notes the consumer's stream (freed_pending); the next
+    // copy that wants any such slot records ONE event per stream for all slots released since, and each of them then
+    // refers to that event (freed_ev) under a ticket that grows with every record.
+    std::vector<hipEvent_t> freed;      // one event object per slot
+    std::vector<char> freed_pending;    // released, no event recorded yet
+    std::vector<hipStream_t> freed_strm;
+    std::vector<hipEvent_t> freed_ev;   // the event the next copy into the slot waits for (some slot's object)
+    std::vector<uint64_t> freed_ticket;
     std::vector<char> freed_valid;
     std::vector<int> order;             // registration order
     std::deque<int> fifo;               // cyclic copy queue
@@ -184,6 +191,12 @@ struct moe_stager {
     int wrap_layers = 0;         // layers [0, wrap_layers) take the last layer as their "previous" one
     int num_hidden_layers = 0, num_local_experts = 0;
     int decoding = 0;
+    int n_held = 0;              // modules acquired and not yet released
+    // Events of one consumer stream are recorded in ticket order, so a wait for ticket T covers every smaller one.
+    // Which ticket the copy stream already waits for, per consumer stream: for copies enqueued by the caller's
+    // thread, and for the bounce worker's jobs (enqueued later, in job order).
+    uint64_t ticket = 0;
+    std::vector<std::pair<hipStream_t, uint64_t>> waited_direct, waited_jobs;
     std::mutex mu;
 };
 
@@ -195,11 +208,56 @@ int find_free(const Type& t) {
     return -1;
 }
 
+// One event per consumer stream for every slot released since the last call.  A wait that is still pending when a
+// copy is enqueued costs the copy stream about 0.2 ms on this runtime: a wave of ten experts released one by one and
+// refilled one by one, each behind its own event, lost 2.3 ms per wave (272 instead of 211 ms per DeepSeek-V3 layer
+// once the host no longer waited for the GPU between waves); with one event per batch of releases the first copy
+// waits and the others are covered by it.
+int flush_released(moe_stager* st) {
+    for (;;) {
+        hipStream_t strm = nullptr;
+        hipEvent_t ev = nullptr;
+        for (Type& t : st->types)
+            for (int s = 0; s < t.n_total; ++s) {
+                if (!t.freed_pending[s]) continue;
+                if (!ev) {
+                    strm = t.freed_strm[s];
+                    ev = t.freed[s];
+                    MOE_HIP_CHECK(hipEventRecord(ev, strm));
+                    ++st->ticket;
+                } else if (t.freed_strm[s] != strm) {
+                    continue;                 // another consumer stream: the next round
+                }
+                t.freed_pending[s] = 0;
+                t.freed_ev[s] = ev;
+                t.freed_ticket[s] = st->ticket;
+                t.freed_valid[s] = 1;
+            }
+        if (!ev) return MOE_OK;
+    }
+}
+
+// whether a wait for `ticket` of consumer stream `strm` is still needed; notes it as issued
+bool need_wait(std::vector<std::pair<hipStream_t, uint64_t>>& waited, hipStream_t strm, uint64_t ticket) {
+    for (auto& w : waited)
+        if (w.first == strm) {
+            if (w.second >= ticket) return false;
+            w.second = ticket;
+            return true;
+        }
+    waited.emplace_back(strm, ticket);
+    return true;
+}
+
 // enqueue the copy of module `id` into free slot `slot` of its type
 int copy_into(moe_stager* st, int id, int slot) {
     Module& m = st->modules[id];
     Type& t = st->types[m.type];
     uint8_t* dst = t.mem + (size_t)slot * t.slot_bytes;
+    if (st->backend == MOE_STAGE_DEVICE && t.freed_pending[slot]) {
+        int rc = flush_released(st);
+        if (rc != MOE_OK) return rc;
+    }
     if (m.pageable) {
         Bounce& b = st->bounce;
         if (b.n_chunks == 0) {
@@ -211,7 +269,7 @@ int copy_into(moe_stager* st, int id, int slot) {
         j.pieces = m.pieces;
         j.ready = m.ready;
         if (st->backend == MOE_STAGE_DEVICE && t.freed_valid[slot]) {
-            j.wait_for = t.freed[slot];
+            if (need_wait(st->waited_jobs, t.freed_strm[slot], t.freed_ticket[slot])) j.wait_for = t.freed_ev[slot];
             t.freed_valid[slot] = 0;
         }
         {
@@ -223,7 +281,8 @@ int copy_into(moe_stager* st, int id, int slot) {
         b.cv_job.notify_one();
     } else if (st->backend == MOE_STAGE_DEVICE) {
         if (t.freed_valid[slot]) {
-            MOE_HIP_CHECK(hipStreamWaitEvent(st->copy_stream, t.freed[slot], 0));
+            if (need_wait(st->waited_direct, t.freed_strm[slot], t.freed_ticket[slot]))
+                MOE_HIP_CHECK(hipStreamWaitEvent(st->copy_stream, t.freed_ev[slot], 0));
             t.freed_valid[slot] = 0;
         }
         for (const Piece& p : m.pieces)
@@ -306,11 +365,13 @@ int release_one(moe_stager* st, int id, hipStream_t stream) {
     Module& m = st->modules[id];
     Type& t = st->types[m.type];
     if (st->backend == MOE_STAGE_DEVICE) {
-        MOE_HIP_CHECK(hipEventRecord(t.freed[m.slot], stream));
-        t.freed_valid[m.slot] = 1;
+        t.freed_pending[m.slot] = 1;
+        t.freed_strm[m.slot] = stream;
+        t.freed_valid[m.slot] = 0;
     }
     t.owner[m.slot] = -1;
     m.slot = -1;
+    if (m.held) --st->n_held;
     m.held = false;
     m.wanted = false;
     return MOE_OK;
@@ -376,6 +437,10 @@ extern "C" int moe_stage_create(moe_stager** out, int32_t n_types, const size_t*
         t.mem = static_cast<uint8_t*>(slot_mem[i]);
         t.owner.assign(t.n_total, -1);
         t.freed.assign(t.n_total, nullptr);
+        t.freed_pending.assign(t.n_total, 0);
+        t.freed_strm.assign(t.n_total, nullptr);
+        t.freed_ev.assign(t.n_total, nullptr);
+        t.freed_ticket.assign(t.n_total, 0);
         t.freed_valid.assign(t.n_total, 0);
     }
     if (backend == MOE_STAGE_DEVICE) {
@@ -505,6 +570,7 @@ extern "C" int moe_stage_acquire(moe_stager* st, int32_t id, void* stream, int32
         if (rc != MOE_OK) return rc;
     }
     if (st->backend == MOE_STAGE_DEVICE) MOE_HIP_CHECK(hipStreamWaitEvent(moe::as_stream(stream), m.ready, 0));
+    if (!m.held) ++st->n_held;
     m.held = true;
     *slot = m.slot;
     return MOE_OK;
@@ -521,7 +587,11 @@ extern "C" int moe_stage_release(moe_stager* st, int32_t id, void* stream) {
     }
     int rc = release_one(st, id, moe::as_stream(stream));
     if (rc != MOE_OK) return rc;
-    int r = pump_all(st);  // the worker refills a freed slot at once
+    // The worker refills a freed slot at once -- on the device once the caller has let go of everything it holds: the
+    // slots of a wave released one after the other then share one event (flush_released).  While other modules
+    // stay held, the refill waits for the next call that copies (acquire, fetch, pump).
+    if (st->backend == MOE_STAGE_DEVICE && st->n_held > 0) return MOE_OK;
+    int r = pump_all(st);
     return r < 0 ? r : MOE_OK;
 }
 

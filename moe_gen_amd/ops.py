@@ -173,36 +173,21 @@ def expert_pointers(gates, ups, downs, s_gates=None, s_ups=None, s_downs=None, d
     return ExpertPointers(E, h, I, fp8, table(gates), table(ups), table(downs), sg, su, sd, keep)
 
 
-class _PinnedRing:
-    """A ring of small pinned host buffers for pointer tables on their way to the device: a table is written into
-    the next buffer and copied with one asynchronous H2D copy; a buffer is reused only after the copy that read it
-    last has completed (its event), which after a trip round the ring it long has."""
-
-    def __init__(self, n_buffers: int = 32, words: int = 8192):
-        self.bufs = [torch.empty(words, dtype=torch.int64, pin_memory=True) for _ in range(n_buffers)]
-        self.views = [b.numpy() for b in self.bufs]
-        self.events = [None] * n_buffers
-        self.i = 0
-        self.words = words
-
-    def push(self, values, device) -> torch.Tensor:
-        n = len(values)
-        if n > self.words:
-            return torch.tensor(values, dtype=torch.int64).to(device)
-        i = self.i
-        self.i = (i + 1) % len(self.bufs)
-        if self.events[i] is not None:
-            self.events[i].synchronize()
-        self.views[i][:n] = values
-        dev = torch.empty(n, dtype=torch.int64, device=device)
-        dev.copy_(self.bufs[i][:n], non_blocking=True)
-        ev = self.events[i] or torch.cuda.Event()
-        ev.record()
-        self.events[i] = ev
-        return dev
+def _upload_words(values, device) -> torch.Tensor:
+    """A device int64 array holding `values`, written by moe_write_words: the words travel in kernel arguments on
+    the current stream: no pinned staging buffer to recycle, and nothing queued on the copy engine behind the weight
+    copies that a stager keeps in flight there."""
+    n = len(values)
+    dev = torch.empty(n, dtype=torch.int64, device=device)
+    arr = (ctypes.c_uint64 * n)(*values)
+    if dev.device.index == torch.cuda.current_device():
+        N.check(N.lib().moe_write_words(dev.data_ptr(), arr, n, _stream()), "moe_write_words")
+    else:
+        with torch.cuda.device(dev.device):
+            N.check(N.lib().moe_write_words(dev.data_ptr(), arr, n, _stream()), "moe_write_words")
+    return dev
 
 
-_rings: dict = {}
 _table_cache: dict = {}       # (device, shape, dtype, pointers) -> ExpertPointers of a wave seen before
 _TABLE_CACHE_MAX = 32768
 
@@ -210,8 +195,9 @@ _TABLE_CACHE_MAX = 32768
 def expert_pointers_of_rows(rows, device) -> ExpertPointers:
     """Pointer tables for one wave of engine-delivered experts: `rows[i]` = (gate, up, down[, s_gate, s_up, s_down])
     of expert i.  The hot form of expert_pointers: shapes and dtypes are checked against the first expert's, all
-    tables travel in ONE pinned, asynchronous copy (six synchronous ones otherwise: 26 waves of a DeepSeek-V3 layer
-    cost 2.4 ms of host time that way), and the tables are slices of that one device array."""
+    tables are written by ONE small launch that carries them in its arguments (six synchronous copies otherwise: 26
+    waves of a DeepSeek-V3 layer cost 2.4 ms of host time that way), and the tables are slices of that one device
+    array."""
     E = len(rows)
     g0, u0, d0 = rows[0][0], rows[0][1], rows[0][2]
     I, h = g0.shape
@@ -241,11 +227,7 @@ def expert_pointers_of_rows(rows, device) -> ExpertPointers:
         for i, r in enumerate(rows):
             if r[3].shape != (bi, bh) or r[4].shape != (bi, bh) or r[5].shape != (bh, bi) or r[3].dtype != torch.float32:
                 raise ValueError(f"experts[{i}]: block scales must be fp32 of shapes {(bi, bh)}, {(bi, bh)}, {(bh, bi)}")
-    key = str(device)
-    ring = _rings.get(key)
-    if ring is None:
-        ring = _rings[key] = _PinnedRing()
-    t = ring.push(vals, device)
+    t = _upload_words(vals, device)
     cols = [t[c * E:(c + 1) * E] for c in range(ncol)]
     out = ExpertPointers(E, h, I, fp8, cols[0], cols[1], cols[2], *(cols[3:] if fp8 else (None, None, None)))
     if len(_table_cache) >= _TABLE_CACHE_MAX:

@@ -353,3 +353,26 @@ def test_segment_to_hbm_through_the_bounce_ring(chunk_bytes):
     copies, nbytes = st.stats()
     assert copies >= 3 * len(mods)
     st.close()
+
+
+@pytest.mark.parametrize("n", [0, 1, 60, 255, 256, 257, 1536])
+def test_write_words_carries_a_pointer_table_in_kernel_arguments(n):
+    """moe_write_words: the words arrive bit for bit, in order, and nothing next to them is touched; the host
+    array may be overwritten as soon as the call has returned (the values travelled with the launch)."""
+    import ctypes
+
+    import numpy as np
+    from moe_gen_amd import _native as N
+
+    rng = np.random.default_rng(n)
+    vals = rng.integers(0, 2**63, size=n, dtype=np.uint64) | (rng.integers(0, 2, size=n, dtype=np.uint64) << np.uint64(63))
+    dev = torch.full((n + 2,), -7, dtype=torch.int64, device="cuda")
+    arr = (ctypes.c_uint64 * max(n, 1))(*[int(v) for v in vals])
+    st = torch.cuda.current_stream().cuda_stream
+    N.check(N.lib().moe_write_words(dev.data_ptr() + 8, arr, n, st), "moe_write_words")
+    for i in range(n):
+        arr[i] = 0
+    got = dev.cpu().numpy().view(np.uint64)
+    assert got[0] == np.uint64(2**64 - 7) and got[-1] == np.uint64(2**64 - 7)
+    assert (got[1:-1] == vals).all()
+    assert N.lib().moe_write_words(dev.data_ptr() + 4, arr, 1, st) != 0      # misaligned destination is refused
