@@ -376,3 +376,46 @@ def test_write_words_carries_a_pointer_table_in_kernel_arguments(n):
     assert got[0] == np.uint64(2**64 - 7) and got[-1] == np.uint64(2**64 - 7)
     assert (got[1:-1] == vals).all()
     assert N.lib().moe_write_words(dev.data_ptr() + 4, arr, 1, st) != 0      # misaligned destination is refused
+
+
+def test_releases_of_a_wave_share_one_event_and_refill_when_nothing_is_held():
+    """Releases only note the consumer's stream; the refills start with the release that leaves nothing held (or
+    with the next call that copies), behind ONE event for the whole batch -- and the slots then hold the right
+    modules' bytes however often the pool has gone round."""
+    from moe_gen_amd import Stager
+    shapes = {"routed_expert": {"w": ((256, 256), torch.bfloat16)}}
+    st = Stager(shapes, {"routed_expert": 4}, model_type="mixtral", num_hidden_layers=4, num_local_experts=12)
+    host = {}
+    for e in range(12):
+        host[e] = torch.randn(256, 256).to(torch.bfloat16).pin_memory()
+        st.add_module(f"routed_expert_0_{e}", "routed_expert", {"w": host[e]})
+    st.pump()
+    assert st.stats()[0] == 4                                   # the pool is full: modules 0-3
+    a = st.get_weights("routed_expert_0_0")["w"]
+    b = st.get_weights("routed_expert_0_1")["w"]
+    assert torch.equal(a.cpu(), host[0]) and torch.equal(b.cpu(), host[1])
+    st.free_weights_buffer("routed_expert_0_0")
+    assert st.stats()[0] == 4                                   # module 1 is still held: no refill yet
+    st.free_weights_buffer("routed_expert_0_1")
+    assert st.stats()[0] == 6                                   # nothing held: both freed slots are refilled (4, 5)
+    # a held module does not stop an explicit pump, or the acquire of a module that needs a slot
+    c = st.get_weights("routed_expert_0_2")["w"]
+    d = st.get_weights("routed_expert_0_3")["w"]
+    st.free_weights_buffer("routed_expert_0_2")
+    assert st.stats()[0] == 6
+    assert st.pump() == 1 and st.stats()[0] == 7                # module 6 into the slot of module 2
+    assert torch.equal(d.cpu(), host[3])
+    st.free_weights_buffer("routed_expert_0_3")
+    # several trips round the pool, two modules at a time, with work on the stream between acquire and release
+    x = torch.zeros(256, 256, device="cuda")
+    order = [4, 5, 6, 7, 8, 9, 10, 11, 0, 1, 2, 3, 4, 5, 6, 7]
+    for i in range(0, len(order), 2):
+        pair = order[i:i + 2]
+        got = [st.get_weights(f"routed_expert_0_{e}")["w"] for e in pair]
+        for e, w in zip(pair, got):
+            x += w.float() @ w.float().t()                       # keeps the slots busy on the stream
+            assert torch.equal(w.cpu(), host[e]), e
+        for e in pair:
+            st.free_weights_buffer(f"routed_expert_0_{e}")
+    st.sync()
+    st.close()
