@@ -24,6 +24,10 @@ def make_experts(E, h, I, fp8, seed):
     return mats
 
 
+def bits_t(t):
+    return t.cpu().view(torch.int16)
+
+
 def f32_of(m):
     if isinstance(m, tuple):
         return O.bf16_to_f32(O.dequant_block(bits(m[0]), m[1].numpy()))
@@ -248,6 +252,44 @@ def test_fp8_weight_streamer_rows_do_not_depend_on_the_tile(h, I):
     wg, wu, wd = (f32_of(m) for m in one)
     ref = O.mlp_f32(O.bf16_to_f32(bits(x)), wg, wu, wd)
     assert rel_max(O.bf16_to_f32(bits(ys[0])), ref) <= TOL
+
+
+@pytest.mark.parametrize("h,I", [(512, 640), (640, 896), (896, 512)])      # 4 / 5 / 7 blocks of 128 k (gate/up), 5 / 7 / 4 (down)
+def test_fp8_weight_streamer_shapes_and_gather(h, I):
+    """The fp8 weight streamer on every token-group count and both sides of each boundary, with block counts that
+    leave 0, 1 and 2 iterations after its loop unrolled by three, rows gathered through row_map, and a down
+    projection whose last N tile is ragged (h = 640, 896)."""
+    counts = [16, 17, 32, 33, 48, 49, 64, 1, 0, 15, 31, 47, 63]
+    print(f"streamer shapes h={h} I={I} counts={counts}", flush=True)
+    y, ref32, refr = run_case(len(counts), h, I, counts, True, seed=61, use_row_map=True)
+    assert np.isfinite(y).all()
+    assert rel_max(y, ref32) <= TOL and rel_max(y, refr) <= TOL
+
+
+def test_fp8_weight_streamer_row_outside_x_reads_zeros():
+    """A row_map entry outside x is a row of zeros for the streamer too (its token DMA goes through a bounds-checked
+    descriptor; such a row and the rows past an expert's last cost no memory request), and its neighbours are
+    untouched: the other rows' bits equal those of a call with valid entries only."""
+    from moe_gen_amd import ops
+    E, h, I, per = 6, 512, 384, 20
+    n = E * per
+    mats = make_experts(E, h, I, True, 5)
+    dm = [[tuple(t.cuda() for t in m) for m in one] for one in mats]
+    ptrs = ops.expert_pointers([o[0][0] for o in dm], [o[1][0] for o in dm], [o[2][0] for o in dm],
+                               [o[0][1] for o in dm], [o[1][1] for o in dm], [o[2][1] for o in dm])
+    x = torch.randn(n, h, generator=torch.Generator().manual_seed(6)).to(torch.bfloat16).cuda()
+    off = torch.arange(0, n + 1, per, dtype=torch.int32).cuda()
+    rm = torch.arange(n, dtype=torch.int32)
+    good = ops.grouped_swiglu(x, rm.cuda(), ptrs, off, n)
+    bad = rm.clone()
+    for r, v in ((7, n), (45, -1), (119, 2**31 - 1)):
+        bad[r] = v
+    got = ops.grouped_swiglu(x, bad.cuda(), ptrs, off, n)
+    torch.cuda.synchronize()
+    keep = torch.ones(n, dtype=torch.bool)
+    keep[[7, 45, 119]] = False
+    assert torch.equal(bits_t(got)[keep], bits_t(good)[keep])
+    assert (got[~keep.cuda()].float() == 0).all()           # SwiGLU of a zero row is zero, and so is its down projection
 
 
 @pytest.mark.parametrize("fp8", [False, True])
