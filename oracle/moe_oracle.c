@@ -21,11 +21,14 @@
  *     expert id.
  *
  * Parity status of every function here: pinned (see tests/test_oracle_*.py:
- * closed forms, brute force, stock torch/numpy library routines), except the
- * Mixtral rules (orc_router with logits_bf16/weights_bf16 and combine mode 2),
- * whose source (transformers==4.42.0, modeling_mixtral.py) is not vendored in
- * the reference tree: "parity unpinned" against the reference text, pinned only
- * against the stock-torch restatement of the published algorithm.
+ * closed forms, brute force, stock torch/numpy library routines).  The Mixtral
+ * rules (orc_router with logits_bf16/weights_bf16 and combine mode 2) follow
+ * transformers==4.42.0, modeling_mixtral.py, which is not vendored in the
+ * reference tree: they are pinned against the stock-torch restatement of the
+ * published algorithm and against the MixtralSparseMoeBlock of the transformers
+ * release that is installed (a later one), except for the one rule that is
+ * specific to 4.42.0 -- routing weights rounded to bf16 before the product --
+ * which is "parity unpinned": it rests on the published source text alone.
  *
  * Build: gcc -O2 -fPIC -shared -ffp-contract=off -fno-fast-math (see Makefile).
  */

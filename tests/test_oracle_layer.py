@@ -70,6 +70,49 @@ def test_mixtral_layer_vs_torch_blocks():
     assert rel_max(O.bf16_to_f32(out)[same], r[same]) <= 1.2e-2
 
 
+def test_mixtral_layer_vs_installed_transformers():
+    """A witness that is not this repository's: the MixtralSparseMoeBlock of the transformers package that happens to
+    be installed (not the reference's pinned 4.42.0, which is absent: the router is the same published algorithm --
+    bf16 gate Linear, softmax in fp32, top-k, renormalisation -- the experts are w1/w3/w2 as gate/up/down with SiLU,
+    and tokens are added expert by expert in ascending id into a bf16 accumulator; newer releases keep the routing
+    weights in fp32 where 4.42.0 rounds them to bf16 first, so outputs are compared to a bound, not bit for bit)."""
+    tf = pytest.importorskip("transformers")
+    mm = pytest.importorskip("transformers.models.mixtral.modeling_mixtral")
+    if not hasattr(mm, "MixtralSparseMoeBlock"):
+        pytest.skip("installed transformers has no MixtralSparseMoeBlock")
+    n, h, I, E, k = 96, 256, 256, 8, 2
+    x, gate, bias, experts, shared, lw = make("mixtral", n, h, I, E, k, False, 3)
+    cfg = tf.MixtralConfig(hidden_size=h, intermediate_size=I, num_local_experts=E, num_experts_per_tok=k,
+                           num_hidden_layers=1, num_attention_heads=4, num_key_value_heads=4, vocab_size=32)
+    blk = mm.MixtralSparseMoeBlock(cfg).to(torch.bfloat16).eval()
+    sd = blk.state_dict()
+    names = set(sd)
+    if {"gate.weight", "experts.gate_up_proj", "experts.down_proj"} <= names:      # fused expert tensors
+        sd["gate.weight"].copy_(gate)
+        sd["experts.gate_up_proj"].copy_(torch.stack([torch.cat([e[0], e[1]], 0) for e in experts]))
+        sd["experts.down_proj"].copy_(torch.stack([e[2] for e in experts]))
+    elif {"gate.weight", "experts.0.w1.weight"} <= names:                          # one module per expert
+        sd["gate.weight"].copy_(gate)
+        for e in range(E):
+            sd[f"experts.{e}.w1.weight"].copy_(experts[e][0])
+            sd[f"experts.{e}.w3.weight"].copy_(experts[e][1])
+            sd[f"experts.{e}.w2.weight"].copy_(experts[e][2])
+    else:
+        pytest.skip(f"unknown parameter layout of the installed MixtralSparseMoeBlock: {sorted(names)[:6]}")
+    with torch.no_grad():
+        got = blk(x.clone())
+    got = (got[0] if isinstance(got, tuple) else got).float().numpy().reshape(n, h)
+    spec = O.RouterSpec.mixtral(E, k)
+    out, aux = O.layer(bits(x).reshape(n, h), lw, spec, O.COMBINE_BF16_SEQ, rounding="ref")
+    tidx = TB.gate_mixtral(x.view(n, h), gate, k)[0].numpy()
+    same = (aux["idx"] == tidx).all(axis=1)               # rows whose bf16-logit ties torch orders the same way
+    assert same.mean() > 0.8
+    assert rel_max(O.bf16_to_f32(out)[same], got[same]) <= 1.2e-2
+    # and the restatement this repository tests against elsewhere agrees with the package on every row
+    ref, _ = TB.mixtral_block(x, gate, experts, k)
+    assert rel_max(ref.float().numpy().reshape(n, h), got) <= 1.2e-2
+
+
 def test_dense_equivalence_k_equals_E():
     """k = E with identical experts and weights summing to 1: the layer is the dense MLP."""
     n, h, I, E = 32, 128, 64, 4
