@@ -344,7 +344,8 @@ int moe_stage_pump(moe_stager* s);
 int moe_stage_acquire(moe_stager* s, int32_t id, void* stream, int32_t* slot);
 /* free_weights_buffer: the slot may be overwritten once `stream` has finished what it was given before this call.
  * The event that says so is recorded on `stream` by the next call that copies into a released slot, one event for
- * all slots released on that stream since the last such call (so `stream` must still exist then); a copy enqueued
+ * all slots released on that stream since the last such call (so `stream` must still exist then; moe_stage_sync
+ * records what is pending, for a caller that is about to destroy a stream); a copy enqueued
  * behind a wait that is still pending costs the copy stream about 0.2 ms, and ten experts released and refilled
  * one by one paid it ten times.  The release that leaves the caller holding no module refills the freed slots at
  * once (the reference's worker refills a slot as soon as it is free, HtoD_Engine.cpp:201-268); while other modules

@@ -390,7 +390,11 @@ int drop_residency(moe_stager* st, int ti, const char* who) {
         int rc = st->bounce.wait_issued(st->bounce.enqueued);
         if (rc != MOE_OK) return rc;
     }
-    if (st->backend == MOE_STAGE_DEVICE) MOE_HIP_CHECK(hipStreamSynchronize(st->copy_stream));
+    if (st->backend == MOE_STAGE_DEVICE) {
+        int rc = flush_released(st);        // (the consumers' streams are named now, while they certainly exist)
+        if (rc != MOE_OK) return rc;
+        MOE_HIP_CHECK(hipStreamSynchronize(st->copy_stream));
+    }
     for (int s = 0; s < t.n_total; ++s) {
         if (t.owner[s] >= 0) {
             st->modules[t.owner[s]].slot = -1;
@@ -763,7 +767,11 @@ extern "C" int moe_stage_sync(moe_stager* st) {
         int rc = st->bounce.wait_issued(st->bounce.enqueued);
         if (rc != MOE_OK) return rc;
     }
-    if (st->backend == MOE_STAGE_DEVICE) MOE_HIP_CHECK(hipStreamSynchronize(st->copy_stream));
+    if (st->backend == MOE_STAGE_DEVICE) {
+        int rc = flush_released(st);
+        if (rc != MOE_OK) return rc;
+        MOE_HIP_CHECK(hipStreamSynchronize(st->copy_stream));
+    }
     return MOE_OK;
 }
 
