@@ -163,8 +163,8 @@ int moe_dispatch_static(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k
  * 64, 128 or (bf16 weights) 192 rows run one workgroup per tile, at a tile height chosen per expert on the device;
  * larger experts run on 256-row tiles of persistent workgroups (with fp8 weights: their full 256-row tiles, and the
  * rows these leave over as one small tile of the first kind if they are at most 128).  The persistent workgroups,
- * one per CU, take whole rounds of tiles; a last round of at most half the CUs' worth of tiles is cut into 128-row
- * halves and runs with the first kind.  Below a mean of 128 rows per expert (n_rows / E), with K not a multiple of
+ * one per CU, take whole rounds of tiles; a last, partial round is cut into 128-row halves and runs with the first
+ * kind when that shortens the two launches (alone: if it is at most half the CUs' worth of tiles).  Below a mean of 128 rows per expert (n_rows / E), with K not a multiple of
  * 128, with more than 512 experts or with 4 GiB or more of gathered x, the one-workgroup-per-tile kernel serves the
  * call alone (larger experts cut into 128-row tiles).  An output row's bits depend on the row and its expert's
  * weights, never on the row's place among its expert's rows or on any expert's count, with one exception: a call

@@ -92,7 +92,7 @@ struct GemmArgs {
                                 // last, ragged one only if it holds more than cold_max rows
     int pair_rows;              // 1: experts of PAIR_LO .. PAIR_HI rows also belong to the one-workgroup-per-tile kernel
     int tail_cus;               // > 0: the persistent kernel runs whole rounds of this many tiles (one per CU); what
-                                // is left, if at most half a round, goes to the other kernel as 128-row half tiles
+                                // is left goes to the other kernel as 128-row half tiles if that pays (tail_tiles)
 };
 
 // LDS rows are 128 bytes = 8 chunks of 16 bytes; chunk c of row r is stored at chunk c ^ swz(r).
@@ -843,11 +843,18 @@ __device__ __forceinline__ int persistent_tiles(const GemmArgs& g, int count) {
 // How many tiles at the end of that space the persistent kernel leaves to the other kernel.  One workgroup per CU
 // walks the space in rounds of tail_cus tiles, and a last round of a few tiles costs as much as a full one while
 // most CUs idle.  Cut into 128-row halves those tiles occupy twice as many CUs for about 0.7 of a tile's time
-// each, which pays if they are at most half a round.  Both kernels evaluate this on the same offsets[].
-__device__ __forceinline__ int tail_tiles(const GemmArgs& g, int total) {
+// each, and they join the other kernel's `own` tiles in its rounds.  The last round moves if that makes the two
+// launches shorter, counting a round of the persistent kernel 1.0 and a round of the other 0.72: alone (own = 0)
+// that is a last round of at most half the CUs; next to other work also a longer one (Mixtral-8x22B, 1024 tokens,
+// down projection: 144 tiles here and 144 there are two half-empty launches in a row, 0.71 ms; as one launch of 432
+// tiles 0.56).  Both kernels evaluate this on the same offsets[].
+__device__ __forceinline__ int tail_tiles(const GemmArgs& g, int total, int own) {
     if (g.tail_cus <= 0) return 0;
-    const int tail = total % g.tail_cus;
-    return 2 * tail <= g.tail_cus ? tail : 0;
+    const int cus = g.tail_cus, tail = total % cus;
+    if (tail == 0) return 0;
+    const int keep = 100 * (total / cus + 1) + 72 * ((own + cus - 1) / cus);
+    const int move = 100 * (total / cus) + 72 * ((own + 2 * tail + cus - 1) / cus);
+    return move < keep ? tail : 0;
 }
 
 template <int SINGLE>   // rows that one tile may hold
@@ -864,6 +871,29 @@ __device__ __forceinline__ int tiles_of(int count) {
 }
 // rows of either tile of such a pair (the first tile holds whole 16-row groups)
 __device__ __forceinline__ int half_rows(int count) { return ((count + 1) / 2 + 15) & ~15; }
+
+// M tiles of an expert with `count` rows in the one-workgroup-per-tile kernel's own tile space
+template <bool W8>
+__device__ __forceinline__ int own_tiles(const GemmArgs& g, int c) {
+    if (g.rem_split) c &= 255;      // the rows the persistent kernel's full tiles leave over
+    return (g.rem_split ? c > g.cold_max : !is_cold(g, c)) ? 0 : tiles_of<(W8 ? 128 : 192)>(c);
+}
+
+// sum over the experts of f(count) (every thread gets it; two barriers)
+template <int NT, typename F>
+__device__ __forceinline__ int sum_over_experts(const GemmArgs& g, int tid, int* s_wtot, F f) {
+    int v = 0;
+    for (int e = tid; e < g.E; e += NT) v += f(g.offsets[e + 1] - g.offsets[e]);
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) v += __shfl_xor(v, d);
+    __syncthreads();                 // whoever read s_wtot before has done so
+    if ((tid & 63) == 0) s_wtot[tid >> 6] = v;
+    __syncthreads();
+    int tot = 0;
+#pragma unroll
+    for (int w = 0; w < NT / 64; ++w) tot += s_wtot[w];
+    return tot;
+}
 
 // One workgroup per (M tile, N tile); serves what the persistent kernel does not take (few rows per expert, odd K).
 template <int WN, bool SWIGLU, bool W8>
@@ -882,10 +912,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     // ---- M-tile prefix over experts ----
     ExpertOfThread mine;
     const bool s8_ok = !g.row_map || g.a_bytes < (1ull << 32);   // (the weight streamer addresses gathered rows with 32-bit offsets)
-    int run = mtile_prefix_scan<NT>(g, tid, s_pref, s_wtot, mine, [&](int c) {
-        if (g.rem_split) c &= 255;      // the rows the persistent kernel's full tiles leave over
-        return (g.rem_split ? c > g.cold_max : !is_cold(g, c)) ? 0 : tiles_of<(W8 ? 128 : 192)>(c);
-    }, [](int, int, int) {});
+    int run = mtile_prefix_scan<NT>(g, tid, s_pref, s_wtot, mine, [&](int c) { return own_tiles<W8>(g, c); }, [](int, int, int) {});
     const int total = run * g.n_tiles_n;
 
     // ---- XCD-aware id: groups of 4 consecutive tiles (the M tiles of one N tile first) go round-robin to the XCDs
@@ -903,7 +930,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
         __syncthreads();                 // s_wtot of the first scan has been read by everyone
         run = mtile_prefix_scan<NT>(g, tid, s_pref, s_wtot, mine, [&](int c) { return persistent_tiles(g, c); }, [](int, int, int) {});
         const int total_p = run * g.n_tiles_n;
-        const int tail = tail_tiles(g, total_p);
+        const int tail = tail_tiles(g, total_p, total);
         if (t >= 2 * tail) return;
         v = total_p - tail + (t >> 1);
         half = t & 1;
@@ -1034,7 +1061,9 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
     });
     if (tid == 0) s_pref[g.E] = run;
     __syncthreads();
-    const int total = run * g.n_tiles_n - tail_tiles(g, run * g.n_tiles_n);   // whole rounds; the rest: the other kernel
+    // whole rounds, and the last one unless it is better off with the other kernel, whose own tiles are counted for that
+    const int own = g.tail_cus > 0 ? sum_over_experts<NT>(g, tid, s_wtot, [&](int c) { return own_tiles<W8>(g, c); }) * g.n_tiles_n : 0;
+    const int total = run * g.n_tiles_n - tail_tiles(g, run * g.n_tiles_n, own);
     const int xcd = blockIdx.x & 7, slots = gridDim.x >> 3;
     int slot = blockIdx.x >> 3;
     auto tile_of = [&](int sl) { return ((sl / slots) * 8 + xcd) * slots + (sl % slots); };
@@ -1292,8 +1321,8 @@ int launch_tiles(const GemmArgs& g, int n_rows, hipStream_t st) {
     auto kern = grouped_gemm_kernel<WN, SWIGLU, W8>;
     // sum_e tiles_of(c_e) <= sum_e (c_e / 128 + 1); with the larger experts elsewhere, one tile per expert that has rows
     const long max_mtiles = g.cold_max <= 192 ? (g.pair_rows ? 2 : 1) * (long)(g.E < n_rows ? g.E : n_rows) : (long)n_rows / 128 + g.E;
-    // (+ the persistent kernel's last tiles, at most half a round of them, as two half tiles each)
-    const long grid = ((max_mtiles * g.n_tiles_n + g.tail_cus + 31) / 32) * 32;   // whole rounds of 8 groups of 4 tiles
+    // (+ the persistent kernel's last tiles, less than a round of them, as two half tiles each)
+    const long grid = ((max_mtiles * g.n_tiles_n + 2 * g.tail_cus + 31) / 32) * 32;   // whole rounds of 8 groups of 4 tiles
     if (grid > 0x7fffffffL) {
         set_error("grouped gemm: %ld workgroups exceed the grid limit", grid);
         return MOE_ERR_INVALID;

@@ -175,14 +175,17 @@ def test_experts_split_between_the_two_kernels(fp8):
 
 
 @pytest.mark.parametrize("fp8", [False, True])
-@pytest.mark.parametrize("I,counts", [(1280, [700, 520, 300, 1300, 90]),      # gate/up: 140 tiles, one partial round
-                                      (2560, [700, 520, 300, 1300, 90]),      # gate/up: 280 tiles, a round + 24
-                                      (1664, [2100, 2300, 2500, 1500, 10])])  # gate/up: 442 tiles, a round + 186
+@pytest.mark.parametrize("I,counts", [(1280, [700, 520, 300, 1300, 90]),      # gate/up: less than half a round
+                                      (2048, [700, 520, 300, 1300, 90]),      # gate/up: 192 tiles next to 48 of the other kernel
+                                      (2560, [700, 520, 300, 1300, 90]),      # gate/up: a round and a few tiles
+                                      (1664, [2100, 2300, 2500, 1500, 10])])  # gate/up: 442 tiles, a round + 186, next to 13
 def test_rounds_of_the_persistent_kernel_and_its_last_tiles(fp8, I, counts):
-    """The persistent kernel (one workgroup per CU) takes whole rounds of 256 tiles; a last round of at most 128
-    tiles goes to the other kernel as 128-row halves, a longer one stays (tile counts in the comments: bf16 weights;
-    with fp8 weights, where only an expert's full tiles and ragged tiles above 128 rows count, 110, 220 and 429).  The
-    down projections of these cases have 14 and 34 tiles, all of them half tiles.  Against the oracle."""
+    """The persistent kernel (one workgroup per CU) takes whole rounds of 256 tiles; its last, partial round goes to
+    the other kernel as 128-row halves when that shortens the two launches: alone, a round of at most 128 tiles;
+    next to the other kernel's own tiles also a longer one (192 + 48 tiles: one launch of 432 half and whole tiles
+    instead of two launches; 186 of 442 likewise).  Tile counts in the comments are for bf16 weights (with fp8
+    weights only an expert's full tiles and ragged tiles above 128 rows count).  The down projections of these cases
+    have a few dozen tiles, all of them half tiles.  Against the oracle."""
     from moe_gen_amd import ops
     E, h = len(counts), 256
     print(f"rounds fp8={fp8} I={I} counts={counts}", flush=True)
