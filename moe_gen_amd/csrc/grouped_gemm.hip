@@ -108,6 +108,7 @@ typedef const __attribute__((address_space(1))) u32x4* gptr_u32x4;
 typedef const __attribute__((address_space(1))) float* gptr_f32;
 typedef const __attribute__((address_space(1))) int32_t* gptr_i32;
 typedef __attribute__((address_space(3))) uint8_t* lds_u8;
+typedef const __attribute__((address_space(4))) float* cptr_f32;   // constant address space: uniform addresses become scalar loads
 
 __device__ __forceinline__ u32x4 gload16(const void* p) { return *(gptr_u32x4)(uintptr_t)p; }
 // Weights under the one-workgroup-per-tile kernel are streamed: a tile of them is used by one workgroup (two
@@ -285,8 +286,15 @@ __device__ __forceinline__ void store_wave_outputs(const f32x4 (&acc)[2 * MT][TN
 // smem0 / smem1: the two LDS stages (two separate arrays: stores into one stage and reads from the other provably
 //     do not alias, which lets the scheduler move them past each other)
 // STREAM: no other tile reads these weights (the expert has one M tile): non-temporal loads
+// One LDS stage of gemm_tile: token rows, weight rows and the start of the region that the epilogue may transpose
+// through (the two parts are one array in the bf16 kernel and separate arrays in the fp8 kernel, whose weight
+// streamers write them by DMA)
+struct Stage {
+    uint8_t *a, *b, *ep;
+};
+
 template <int MT, int WN, bool SWIGLU, bool W8, bool STREAM>
-__device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uint8_t* smem1, int e, int row0, int row_end,
+__device__ __forceinline__ void gemm_tile(const GemmArgs& g, Stage st0, Stage st1, int e, int row0, int row_end,
                                           int n_tile) {
     constexpr int NT = 128 * WN;                // threads
     constexpr int BM = 64 * MT;                 // rows per workgroup
@@ -414,8 +422,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
             rb[set][i] = gload16_w<STREAM>(m + ((size_t)b_n[i] * K + kofs) * 2 + bcol_b);
         }
     };
-    auto lds_store = [&](uint8_t* As, int set) {
-        uint8_t* Bs = As + A_STAGE;
+    auto lds_store = [&](Stage S, int set) {
+        uint8_t *As = S.a, *Bs = S.b;
 #pragma unroll
         for (int i = 0; i < NA; ++i) *reinterpret_cast<u32x4*>(As + a_lds + i * RA * ROW_B) = a_ok[i] ? ra[set][i] : u32x4{0, 0, 0, 0};
         if (PAIR8) {
@@ -469,13 +477,14 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
     bool live[TM];
 #pragma unroll
     for (int mi = 0; mi < TM; ++mi) live[mi] = wm * 32 * MT + 16 * mi < row_end - row0;
-    auto read_w1 = [&](const uint8_t* As, int s, int j, auto part) __attribute__((always_inline)) {
+    auto read_w1 = [&](Stage S, int s, int j, auto part) __attribute__((always_inline)) {
         if (decltype(part)::value && !live[0]) return;
-        const uint8_t* Bs = As + A_STAGE;
+        const uint8_t* Bs = S.b;
         const uint32_t coff = (uint32_t)(((4 * s + fchunk) ^ fkey) << 4);
         wfr[s][j] = *reinterpret_cast<const bf16x8*>(Bs + w_off[j] + coff);
     };
-    auto read_tq = [&](const uint8_t* As, int u, auto part) __attribute__((always_inline)) {
+    auto read_tq = [&](Stage S, int u, auto part) __attribute__((always_inline)) {
+        const uint8_t* As = S.a;
         const int s = u / NP, q = u % NP;
         const uint32_t coff = (uint32_t)(((4 * s + fchunk) ^ fkey) << 4);
 #pragma unroll
@@ -507,7 +516,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
 #pragma unroll
         for (int i = 0; i < 4; ++i) pair_load(1, 1, i);
     }
-    lds_store(smem0, 0);
+    lds_store(st0, 0);
     // No load or store of the pipeline sits under a branch or in a region that only some waves
     // execute (past the end the last tile is loaded again and stored where nobody reads it): with
     // straight-line code the compiler counts the outstanding loads exactly, so a store waits only
@@ -524,8 +533,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
     // waits each item stalls only until its own chunk (requested PF iterations earlier) is there.
     constexpr int NI = NA + NB;
     // par = kt & 1 and ps, the register set of the pair that stage kt+1 belongs to, are literals at the call sites
-    auto data_item = [&](int i, uint8_t* As, int kt, int set, int par, int ps) __attribute__((always_inline)) {
-        uint8_t* Bs = As + A_STAGE;
+    auto data_item = [&](int i, Stage S, int kt, int set, int par, int ps) __attribute__((always_inline)) {
+        uint8_t *As = S.a, *Bs = S.b;
         const int kn = stage_at(min(kt + 1 + PF, nk - 1));
         const size_t kofs = (size_t)kn * BK;
         // past the end nobody reads what is loaded: streamed weights would come from HBM once more
@@ -553,8 +562,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
     constexpr int NG = NU;                        // one group of MFMAs per slot
     constexpr int WPS = TN / NP;                  // weight fragments of the second k-step read per slot
     auto iteration = [&](int kt, int set, int par, int ps, auto part) __attribute__((always_inline)) {   // par == kt & 1
-        const uint8_t* rd = par ? smem1 : smem0;
-        uint8_t* wr = par ? smem0 : smem1;
+        const Stage rd = par ? st1 : st0;
+        const Stage wr = par ? st0 : st1;
 #pragma unroll
         for (int v = 0; v < NU; ++v) {
             // group v takes items [v*NI/NG, (v+1)*NI/NG): in order, so the two halves of an fp8
@@ -617,7 +626,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, uint8_t* smem0, uin
     // All waves passed the loop's last barrier, so no one reads the stages: each wave transposes through its own
     // slice of them.
     constexpr int CW = SWIGLU ? 8 * TN : 16 * TN;    // output columns of this wave
-    uint8_t* ep = ((wave < 4) ? smem0 : smem1) + (wave & 3) * (32 * MT * CW * 2);
+    uint8_t* ep = ((wave < 4) ? st0.ep : st1.ep) + (wave & 3) * (32 * MT * CW * 2);
     const int ncol0 = n0 + wn * CW;
     store_wave_outputs<MT, TN, SWIGLU, 32 * MT, false>(acc, ep, lane, g.c + (size_t)(row0 + wm * 32 * MT) * N + ncol0, N,
                                                        min(BM, row_end - row0) - wm * 32 * MT, N - ncol0);
@@ -652,8 +661,14 @@ constexpr int S8_WBYTES = 32 * 1024;              // weight region of a buffer: 
 constexpr int S8_TROWS = 64;                      // token rows staged
 constexpr int S8_BUF = S8_WBYTES + S8_TROWS * 256;
 
+// A buffer of the weight streamers: the weight region and the token region are separate LDS arrays, so that a read of
+// one never has to wait for a DMA into the other
+struct SBuf {
+    uint8_t *w, *t;
+};
+
 template <int TG, bool SWIGLU>   // TG: 16-row token groups multiplied (the expert has at most 16 TG <= 64 rows)
-__device__ __forceinline__ void stream8_tile(const GemmArgs& g, uint8_t* buf0, uint8_t* buf1, uint8_t* buf2, int e, int row0,
+__device__ __forceinline__ void stream8_tile(const GemmArgs& g, SBuf buf0, SBuf buf1, SBuf buf2, int e, int row0,
                                              int row_end, int n_tile) {
     constexpr int NBLK = SWIGLU ? 128 : 256;
     constexpr int NDW = 4, NDT = 2;               // DMA instructions per wave and 128-k block: weights, tokens
@@ -717,7 +732,7 @@ __device__ __forceinline__ void stream8_tile(const GemmArgs& g, uint8_t* buf0, u
     };
     // DMA instruction i of a block: 0 .. NDW-1 weights (read once: non-temporal, which is worth 5 % of the stream),
     // NDW .. NDW+NDT-1 tokens
-    auto dma_one = [&](int p_pipe, uint8_t* buf, int i) __attribute__((always_inline)) {
+    auto dma_one = [&](int p_pipe, SBuf buf, int i) __attribute__((always_inline)) {
         // past the end of k nobody reads what arrives: an empty descriptor returns zeros without touching memory,
         // and the instruction still counts
         const int live = uni(p_pipe < npair ? -1 : 0);   // (a scalar, or the descriptor ends up in vector registers)
@@ -725,14 +740,14 @@ __device__ __forceinline__ void stream8_tile(const GemmArgs& g, uint8_t* buf0, u
         pr = pr >= npair ? pr - npair : pr;
         if (i < NDW) {
             const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)bmat[i >> 1], 0, live, 0x00020000);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_u8)(buf + wave * 4096 + i * 1024), 16, w_voff[i], (uint32_t)(pr * 128), 0, 2);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_u8)(buf.w + wave * 4096 + i * 1024), 16, w_voff[i], (uint32_t)(pr * 128), 0, 2);
         } else {
             const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)a_base, 0, live & a_records, 0x00020000);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_u8)(buf + S8_WBYTES + wave * 2048 + (i - NDW) * 1024), 16, t_voff[i - NDW],
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_u8)(buf.t + wave * 2048 + (i - NDW) * 1024), 16, t_voff[i - NDW],
                                                      (uint32_t)(pr * 256), 0, 0);
         }
     };
-    auto dma = [&](int p_pipe, uint8_t* buf) {
+    auto dma = [&](int p_pipe, SBuf buf) {
 #pragma unroll
         for (int i = 0; i < NDW + NDT; ++i) dma_one(p_pipe, buf, i);
     };
@@ -740,7 +755,7 @@ __device__ __forceinline__ void stream8_tile(const GemmArgs& g, uint8_t* buf0, u
     const int frow = lane & 15, q = lane >> 4;
     const int fq = ((q & 1) << 1) | (q >> 1);
     const uint32_t w_rd = (uint32_t)(wave * 4096 + frow * 128), wkey = (uint32_t)wsw(frow);
-    const uint32_t t_rd = (uint32_t)(S8_WBYTES + frow * 256), tkey = (uint32_t)tsw(frow);   // (group bases are multiples of 16)
+    const uint32_t t_rd = (uint32_t)(frow * 256), tkey = (uint32_t)tsw(frow);   // (group bases are multiples of 16)
     f32x4 acc[TG][2];
 #pragma unroll
     for (int t = 0; t < TG; ++t) { acc[t][0] = f32x4{0}; acc[t][1] = f32x4{0}; }
@@ -750,7 +765,7 @@ __device__ __forceinline__ void stream8_tile(const GemmArgs& g, uint8_t* buf0, u
     // would make the compiler wait for ALL outstanding DMA).  After the barrier every wave has left block p - 1,
     // whose buffer takes block p + 2 (its DMA is spread over the iteration).  The scale loads come BEFORE the DMA: the
     // compiler's own wait for a scale counts everything issued after it as allowed to be in flight.
-    auto iteration = [&](int p, const uint8_t* rd, uint8_t* refill, int sset) __attribute__((always_inline)) {
+    auto iteration = [&](int p, SBuf rd, SBuf refill, int sset) __attribute__((always_inline)) {
         // (lgkmcnt: this wave's LDS reads of block p - 1 have returned -- its last matrix instructions may be scheduled
         // behind the barrier, and the buffer they read is refilled right after it)
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" :: "n"(VM_BLOCK) : "memory");
@@ -763,7 +778,7 @@ __device__ __forceinline__ void stream8_tile(const GemmArgs& g, uint8_t* buf0, u
             bf16x8 wa[2][2];
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const u32x4 raw = *reinterpret_cast<const u32x4*>(rd + w_rd + j * 2048 + (((4 * h + fq) ^ wkey) << 4));
+                const u32x4 raw = *reinterpret_cast<const u32x4*>(rd.w + w_rd + j * 2048 + (((4 * h + fq) ^ wkey) << 4));
                 wa[j][0] = __builtin_bit_cast(bf16x8, dequant8(raw[0], raw[1], rsc[sset][j]));
                 wa[j][1] = __builtin_bit_cast(bf16x8, dequant8(raw[2], raw[3], rsc[sset][j]));
             }
@@ -772,7 +787,7 @@ __device__ __forceinline__ void stream8_tile(const GemmArgs& g, uint8_t* buf0, u
                 const uint32_t coff = (uint32_t)(((8 * h + 2 * fq + s2) ^ tkey) << 4);
 #pragma unroll
                 for (int t = 0; t < TG; ++t) {
-                    const bf16x8 tf = *reinterpret_cast<const bf16x8*>(rd + t_rd + t * 16 * 256 + coff);
+                    const bf16x8 tf = *reinterpret_cast<const bf16x8*>(rd.t + t_rd + t * 16 * 256 + coff);
                     acc[t][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[0][s2], tf, acc[t][0], 0, 0, 0);
                     acc[t][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[1][s2], tf, acc[t][1], 0, 0, 0);
                 }
@@ -803,6 +818,191 @@ __device__ __forceinline__ void stream8_tile(const GemmArgs& g, uint8_t* buf0, u
     if (p < npair) {
         iteration(p, buf0, buf2, 0);
         if (p + 1 < npair) iteration(p + 1, buf1, buf0, 1);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no DMA may land in LDS after the workgroup has gone
+
+    // ---- epilogue: a lane holds 4 consecutive columns of one row per accumulator and stores them itself ----
+#pragma unroll
+    for (int t = 0; t < TG; ++t) {
+        const int r = row0 + 16 * t + frow;
+        if (r >= row_end) continue;
+        if (SWIGLU) {
+            const int col = n0 + 16 * wave + 4 * q;
+            if (col < N) *reinterpret_cast<u32x2*>(g.c + (size_t)r * N + col) = epilogue_pack<true>(acc[t][0], acc[t][1]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int col = n0 + 32 * wave + 16 * j + 4 * q;
+                if (col < N) *reinterpret_cast<u32x2*>(g.c + (size_t)r * N + col) = epilogue_pack<false>(acc[t][j], acc[t][j]);
+            }
+        }
+    }
+}
+
+
+// ---- fp8 weight streamer in the persistent kernel's summation order: tiles of up to 128 rows ----
+//
+// The same division of labour as stream8_tile (8 waves x 32 weight rows, fp8 weights by DMA in whole lines, every wave
+// multiplies all token rows), for tiles whose rows another kernel might have computed: what an fp8 expert's full
+// 256-row tiles leave over, the halves of the persistent kernel's last tiles, and in calls that this kernel serves
+// alone the experts (or 128-row slices of experts) above 64 rows.  A row's bits must then not depend on who computes
+// it, so every matrix instruction gets the k values the persistent kernel gives it, in the same lanes: lane group q
+// holds k = 32 s + 8 f(q) + (0..7) of k-step s, f = 0, 2, 1, 3.  Those are 8 consecutive fp8 weights, one ds_read_b64
+// (two per 16-byte DMA chunk; the weights are a ninth of the LDS reads), and the 16-byte token chunk 4 s + f(q) of a
+// 64-k half.  128 token rows x 128 k would not fit LDS three times over next to the weights, so token rows travel in
+// halves of 64 k (128 rows x 128 bytes = 16 KiB) through three buffers of their own, one barrier per half, while the
+// weights keep their three buffers of 128 k: 96 + 48 KiB.  Per half-block a wave issues 2 weight DMA instructions (of
+// the block two ahead) and 2 token DMA instructions (of the half two ahead), and the wait before a half's barrier
+// leaves the 4 of the half before in flight.  k starts at block 0 unless the kernel has the call to itself.
+template <int TG, bool SWIGLU>   // TG: 16-row token groups multiplied (1 .. 8)
+__device__ __forceinline__ void stream8x_tile(const GemmArgs& g, SBuf b0, SBuf b1, SBuf b2, int e, int row0, int row_end,
+                                              int n_tile, bool rotate) {
+    constexpr int NBLK = SWIGLU ? 128 : 256;
+    constexpr int VM_HALF = 4;                    // DMA instructions per wave and half-block: 2 weights + 2 tokens
+    static_assert(TG >= 1 && TG <= 8, "token rows staged");
+    const int tid = threadIdx.x, lane = tid & 63, wave = uni(tid >> 6);
+    const int n0 = n_tile * NBLK;
+    const int K = g.K, N = g.N;
+    const int npair = K >> 7;
+    const int prot = rotate ? n_tile % npair : 0;
+
+    // ---- DMA coordinates ----
+    // weights, instruction i (0..3): rows 8 i + lane / 8 of the wave's 32 (fragment i / 2, fragment row 8 (i & 1) + lane / 8);
+    // 16-byte part c of fragment row r at part c ^ wsw(r)
+    const int lr = lane >> 3, pp = lane & 7;
+    uint32_t w_voff[4];
+    const uint8_t* bmat[2];
+    cptr_f32 sc[2];
+    int srow[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        bmat[j] = uni_ptr((SWIGLU && j == 1) ? g.b1[e] : g.b0[e]);
+        sc[j] = (cptr_f32)(uintptr_t)uni_ptr((SWIGLU && j == 1) ? g.s1[e] : g.s0[e]);
+        srow[j] = min((n0 + (SWIGLU ? 0 : 32 * wave)) >> 7, (N >> 7) - 1) * npair;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int fr = 8 * (i & 1) + lr;
+        const int rt = SWIGLU ? 16 * wave + fr : 32 * wave + 16 * (i >> 1) + fr;      // row of the tile's N range
+        w_voff[i] = (uint32_t)min(n0 + rt, N - 1) * (uint32_t)K + (uint32_t)((pp ^ wsw(fr)) << 4);
+    }
+    // tokens, instruction i (0..1): rows 16 wave + 8 i + lane / 8 of the 128 staged, 16-byte chunk c of row r at chunk
+    // c ^ swz(r) (the persistent kernel's layout of a 64-k stage).  Rows past the tile's last: zeros, no request.
+    uint32_t t_voff[2];
+    const uint8_t* a_base = reinterpret_cast<const uint8_t*>(g.a) + (g.row_map ? (size_t)0 : (size_t)row0 * K * 2);
+    const int a_records = g.row_map ? (int)(uint32_t)g.a_bytes : (row_end - row0) * K * 2;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int tr = 16 * wave + 8 * i + lr;
+        const int r = min(row0 + tr, row_end - 1);
+        const int src = g.row_map ? ((gptr_i32)(uintptr_t)g.row_map)[r] : r - row0;
+        t_voff[i] = (uint32_t)src * (uint32_t)(K * 2) + (uint32_t)((pp ^ swz(tr)) << 4);
+        if (row0 + tr >= row_end || (g.row_map && (unsigned)src >= (unsigned)g.a_rows)) t_voff[i] = 0xfffffff0u;
+    }
+    float rsc[2][2];                              // block scales of the block being multiplied / of the next one
+    auto scales = [&](int p_pipe, int set) {      // scalar loads (uniform addresses in the constant address space)
+        int pr = min(p_pipe, npair - 1) + prot;
+        pr = pr >= npair ? pr - npair : pr;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) rsc[set][j] = sc[j][srow[j] + pr];
+    };
+    // weight DMA instruction i of block p_pipe (pipeline order) / token DMA instruction i of half-block hb_pipe
+    auto dma_w = [&](int p_pipe, SBuf buf, int i) __attribute__((always_inline)) {
+        const int live = uni(p_pipe < npair ? -1 : 0);   // past the end: an empty descriptor, zeros without a request
+        int pr = min(p_pipe, npair - 1) + prot;
+        pr = pr >= npair ? pr - npair : pr;
+        const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)bmat[i >> 1], 0, live, 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_u8)(buf.w + wave * 4096 + i * 1024), 16, w_voff[i], (uint32_t)(pr * 128), 0, 2);
+    };
+    auto dma_t = [&](int hb_pipe, SBuf buf, int i) __attribute__((always_inline)) {
+        const int live = uni(hb_pipe < 2 * npair ? -1 : 0);
+        const int hb = min(hb_pipe, 2 * npair - 1);
+        int pr = (hb >> 1) + prot;
+        pr = pr >= npair ? pr - npair : pr;
+        const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)a_base, 0, live & a_records, 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_u8)(buf.t + wave * 2048 + i * 1024), 16, t_voff[i],
+                                                 (uint32_t)(pr * 256 + (hb & 1) * 128), 0, 0);
+    };
+
+    const int frow = lane & 15, q = lane >> 4;
+    const int fq = ((q & 1) << 1) | (q >> 1);
+    // weights: the 8 bytes at 32 s + 8 f(q) of the 64-byte half h of fragment row frow: 16-byte part 4 h + 2 s + f(q) / 2
+    const uint32_t w_rd = (uint32_t)(wave * 4096 + frow * 128 + (fq & 1) * 8), wkey = (uint32_t)wsw(frow);
+    const uint32_t t_rd = (uint32_t)(frow * 128), tkey = (uint32_t)swz(frow);   // (group bases are multiples of 16 rows)
+    f32x4 acc[TG][2];
+#pragma unroll
+    for (int t = 0; t < TG; ++t) { acc[t][0] = f32x4{0}; acc[t][1] = f32x4{0}; }
+
+    // Half-block H = 2 p + h multiplies half h of block p: weights out of buffer p % 3, tokens out of token buffer
+    // H % 3.  Before it: this wave's DMA of its tokens (issued two halves ago) and of everything older has landed and
+    // its LDS reads have returned, then everybody's (a bare s_barrier).  After the barrier every wave has left half
+    // H - 1, whose token buffer takes half H + 2, and (h == 0) block p - 1, whose weight buffer takes block p + 2 over
+    // the two halves of block p.
+    auto half = [&](int p, int h, SBuf wb, SBuf tb, SBuf w_refill, SBuf t_refill, int sset) __attribute__((always_inline)) {
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" :: "n"(VM_HALF) : "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        // every operand of the half is requested up front (2 + TG reads per k-step): the matrix instructions then run
+        // behind the LDS pipeline instead of waiting out its latency one token group at a time
+        u32x2 wraw[2][2];
+        bf16x8 tf[2][TG];
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                wraw[s2][j] = *reinterpret_cast<const u32x2*>(wb.w + w_rd + j * 2048 + (((4 * h + 2 * s2 + (fq >> 1)) ^ wkey) << 4));
+            const uint32_t coff = (uint32_t)(((4 * s2 + fq) ^ tkey) << 4);
+#pragma unroll
+            for (int t = 0; t < TG; ++t) tf[s2][t] = *reinterpret_cast<const bf16x8*>(tb.t + t_rd + t * 16 * 128 + coff);
+        }
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            bf16x8 wa[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) wa[j] = __builtin_bit_cast(bf16x8, dequant8(wraw[s2][j][0], wraw[s2][j][1], rsc[sset][j]));
+#pragma unroll
+            for (int t = 0; t < TG; ++t) {
+                acc[t][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[0], tf[s2][t], acc[t][0], 0, 0, 0);
+                acc[t][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[1], tf[s2][t], acc[t][1], 0, 0, 0);
+            }
+            dma_w(p + 2, w_refill, 2 * h + s2);
+            dma_t(2 * p + h + 2, t_refill, s2);
+        }
+        // (the next block's scales: scalar loads, issued where no LDS read is outstanding -- the two share a counter
+        // and scalar loads return out of order, which would turn every operand wait into a full drain)
+        if (h == 0) scales(p + 1, sset ^ 1);
+    };
+    // Prologue: blocks 0 and 1 and halves 0 and 1, the tokens of half 0 before the weights of block 1, so that the
+    // first half's wait (all but the 4 youngest instructions) covers what it reads, as in the steady state.
+    scales(0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_w(0, b0, i);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) dma_t(0, b0, i);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_w(1, b1, i);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) dma_t(1, b1, i);
+    // Six halves = three blocks bring both rotations back to where they started: literal buffers in the loop body.
+    int p = 0;
+    for (; p + 3 <= npair; p += 3) {
+        half(p, 0, b0, b0, b2, b2, 0);
+        half(p, 1, b0, b1, b2, b0, 0);
+        half(p + 1, 0, b1, b2, b0, b1, 1);
+        half(p + 1, 1, b1, b0, b0, b2, 1);
+        half(p + 2, 0, b2, b1, b1, b0, 0);
+        half(p + 2, 1, b2, b2, b1, b1, 0);
+        const float t0 = rsc[0][0], t1 = rsc[0][1];
+        rsc[0][0] = rsc[1][0]; rsc[0][1] = rsc[1][1];
+        rsc[1][0] = t0; rsc[1][1] = t1;
+    }
+    if (p < npair) {
+        half(p, 0, b0, b0, b2, b2, 0);
+        half(p, 1, b0, b1, b2, b0, 0);
+        if (p + 1 < npair) {
+            half(p + 1, 0, b1, b2, b0, b1, 1);
+            half(p + 1, 1, b1, b0, b0, b2, 1);
+        }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no DMA may land in LDS after the workgroup has gone
 
@@ -895,15 +1095,40 @@ __device__ __forceinline__ int sum_over_experts(const GemmArgs& g, int tid, int*
     return tot;
 }
 
+template <bool SWIGLU>
+__device__ __forceinline__ void stream8x(const GemmArgs& g, SBuf b0, SBuf b1, SBuf b2, int e, int row0, int row_end, int n_tile,
+                                         bool rotate) {
+    const int rows = row_end - row0;
+    if (rows <= 16) stream8x_tile<1, SWIGLU>(g, b0, b1, b2, e, row0, row_end, n_tile, rotate);
+    else if (rows <= 32) stream8x_tile<2, SWIGLU>(g, b0, b1, b2, e, row0, row_end, n_tile, rotate);
+    else if (rows <= 48) stream8x_tile<3, SWIGLU>(g, b0, b1, b2, e, row0, row_end, n_tile, rotate);
+    else if (rows <= 64) stream8x_tile<4, SWIGLU>(g, b0, b1, b2, e, row0, row_end, n_tile, rotate);
+    else if (rows <= 80) stream8x_tile<5, SWIGLU>(g, b0, b1, b2, e, row0, row_end, n_tile, rotate);
+    else if (rows <= 96) stream8x_tile<6, SWIGLU>(g, b0, b1, b2, e, row0, row_end, n_tile, rotate);
+    else if (rows <= 112) stream8x_tile<7, SWIGLU>(g, b0, b1, b2, e, row0, row_end, n_tile, rotate);
+    else stream8x_tile<8, SWIGLU>(g, b0, b1, b2, e, row0, row_end, n_tile, rotate);
+}
+
 // One workgroup per (M tile, N tile); serves what the persistent kernel does not take (few rows per expert, odd K).
 template <int WN, bool SWIGLU, bool W8>
 __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     constexpr int NT = 128 * WN;
-    constexpr int STAGE_MAX = ((W8 ? 128 : 192) + BN_ROWS) * ROW_B;   // a stage of the tallest tile
-    __shared__ __attribute__((aligned(1024))) uint8_t smem0[STAGE_MAX];
-    __shared__ __attribute__((aligned(1024))) uint8_t smem1[STAGE_MAX];
-    __shared__ __attribute__((aligned(1024))) uint8_t smem2[W8 ? S8_BUF : 16];   // third buffer of the fp8 weight streamer
-    static_assert(!W8 || STAGE_MAX >= S8_BUF, "the streamer's buffers are the two stages and a third array");
+    // bf16 weights: two stages of the tallest tile (192 token rows + 256 weight rows).  fp8 weights: three weight
+    // arrays of 32 KiB and three token arrays of 16 KiB -- the buffers of the weight streamers, written by DMA, as
+    // separate objects so that a read of one waits for no DMA into another; gemm_tile's two stages (128 + 256 rows)
+    // are two pairs of them.
+    constexpr int WB = W8 ? S8_WBYTES : (192 + BN_ROWS) * ROW_B;
+    constexpr int TB = W8 ? 128 * ROW_B : 16;
+    __shared__ __attribute__((aligned(1024))) uint8_t lw0[WB];
+    __shared__ __attribute__((aligned(1024))) uint8_t lw1[WB];
+    __shared__ __attribute__((aligned(1024))) uint8_t lw2[W8 ? S8_WBYTES : 16];
+    __shared__ __attribute__((aligned(1024))) uint8_t lt0[TB];
+    __shared__ __attribute__((aligned(1024))) uint8_t lt1[TB];
+    __shared__ __attribute__((aligned(1024))) uint8_t lt2[TB];
+    static_assert(S8_TROWS * 256 <= 128 * ROW_B, "token region of a streamer buffer");
+    auto stage = [&](int i, int mt) { return W8 ? Stage{i ? lt1 : lt0, i ? lw1 : lw0, i ? lw1 : lw0}
+                                                 : Stage{i ? lw1 : lw0, (i ? lw1 : lw0) + 64 * mt * ROW_B, i ? lw1 : lw0}; };
+    const SBuf sb0{lw0, lt0}, sb1{lw1, lt1}, sb2{lw2, lt2};
     __shared__ int s_pref[MAX_E + 1];
     __shared__ int s_wtot[NT / 64];
     __shared__ int s_sel[5];
@@ -966,29 +1191,38 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     if (half >= 0) {                     // half of a 256-row tile of the persistent kernel's space
         const int r0 = uni(s_sel[3]) + m_tile * 256 + half * 128;
         const int r1 = min(uni(s_sel[4]), uni(s_sel[3]) + (m_tile + 1) * 256);
-        if (r0 < r1) gemm_tile<2, WN, SWIGLU, W8, false>(g, smem0, smem1, e, r0, r1, n_tile);
+        if (r0 >= r1) return;
+        if (W8 && s8_ok) stream8x<SWIGLU>(g, sb0, sb1, sb2, e, r0, r1, n_tile, false);
+        else gemm_tile<2, WN, SWIGLU, W8, false>(g, stage(0, 2), stage(1, 2), e, r0, r1, n_tile);
         return;
     }
     const int row_end = uni(s_sel[4]);
     const int first_row = uni(s_sel[3]) + (g.rem_split ? ((row_end - uni(s_sel[3])) & ~255) : 0);
-    if (W8 && g.cold_max == 0x7fffffff && row_end - first_row <= 64 && s8_ok) {
-        // (this kernel has the call to itself, so no other kernel's summation order has to be matched.  An expert of
-        // 65 to 128 rows as two such tiles on neighbouring workgroups measured slower than one 128-row tile of
-        // gemm_tile: 2.99 against 3.68 TB/s of weights at 96 rows per expert.)
-        const int rows = row_end - first_row;
-        if (rows <= 16) stream8_tile<1, SWIGLU>(g, smem0, smem1, smem2, e, first_row, row_end, n_tile);
-        else if (rows <= 32) stream8_tile<2, SWIGLU>(g, smem0, smem1, smem2, e, first_row, row_end, n_tile);
-        else if (rows <= 48) stream8_tile<3, SWIGLU>(g, smem0, smem1, smem2, e, first_row, row_end, n_tile);
-        else stream8_tile<4, SWIGLU>(g, smem0, smem1, smem2, e, first_row, row_end, n_tile);
+    const bool alone = g.cold_max == 0x7fffffff;
+    if (W8 && s8_ok) {
+        // fp8 weights: the weight streamers.  Up to 64 rows in a call that this kernel has to itself, where no other
+        // kernel's summation order has to be matched: the form that reads a lane's 16 weights at once.  Everything
+        // else -- up to 128 rows; what an expert's full 256-row tiles leave over; 128-row slices of larger experts
+        // when the kernel is alone -- in the persistent kernel's order.
+        const int r0 = first_row + (mt_e > 1 ? m_tile * 128 : 0), r1 = mt_e > 1 ? min(row_end, r0 + 128) : row_end;
+        const int rows = r1 - r0;
+        if (alone && mt_e == 1 && rows <= 64) {
+            if (rows <= 16) stream8_tile<1, SWIGLU>(g, sb0, sb1, sb2, e, r0, r1, n_tile);
+            else if (rows <= 32) stream8_tile<2, SWIGLU>(g, sb0, sb1, sb2, e, r0, r1, n_tile);
+            else if (rows <= 48) stream8_tile<3, SWIGLU>(g, sb0, sb1, sb2, e, r0, r1, n_tile);
+            else stream8_tile<4, SWIGLU>(g, sb0, sb1, sb2, e, r0, r1, n_tile);
+        } else {
+            stream8x<SWIGLU>(g, sb0, sb1, sb2, e, r0, r1, n_tile, alone);
+        }
         return;
     }
-    if (row_end - first_row <= 64) gemm_tile<1, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
-    else if (row_end - first_row <= 128) gemm_tile<2, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
-    else if (!W8 && mt_e == 1) gemm_tile<3, WN, SWIGLU, W8, true>(g, smem0, smem1, e, first_row, row_end, n_tile);
+    if (row_end - first_row <= 64) gemm_tile<1, WN, SWIGLU, W8, true>(g, stage(0, 1), stage(1, 1), e, first_row, row_end, n_tile);
+    else if (row_end - first_row <= 128) gemm_tile<2, WN, SWIGLU, W8, true>(g, stage(0, 2), stage(1, 2), e, first_row, row_end, n_tile);
+    else if (!W8 && mt_e == 1) gemm_tile<3, WN, SWIGLU, W8, true>(g, stage(0, 3), stage(1, 3), e, first_row, row_end, n_tile);
     else if (!W8 && row_end - first_row >= PAIR_LO && row_end - first_row <= PAIR_HI) {
         const int r0 = first_row + m_tile * half_rows(row_end - first_row);
-        gemm_tile<3, WN, SWIGLU, W8, false>(g, smem0, smem1, e, r0, min(row_end, r0 + half_rows(row_end - first_row)), n_tile);
-    } else gemm_tile<2, WN, SWIGLU, W8, false>(g, smem0, smem1, e, first_row + m_tile * 128, row_end, n_tile);
+        gemm_tile<3, WN, SWIGLU, W8, false>(g, stage(0, 3), stage(1, 3), e, r0, min(row_end, r0 + half_rows(row_end - first_row)), n_tile);
+    } else gemm_tile<2, WN, SWIGLU, W8, false>(g, stage(0, 2), stage(1, 2), e, first_row + m_tile * 128, row_end, n_tile);
 }
 
 // lane id produced where it is used: the compiler cannot hoist it (and everything derived from it)
