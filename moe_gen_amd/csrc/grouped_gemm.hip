@@ -847,8 +847,8 @@ __device__ __forceinline__ void stream8_tile(const GemmArgs& g, SBuf buf0, SBuf 
 // 256-row tiles leave over, the halves of the persistent kernel's last tiles, and in calls that this kernel serves
 // alone the experts (or 128-row slices of experts) above 64 rows.  A row's bits must then not depend on who computes
 // it, so every matrix instruction gets the k values the persistent kernel gives it, in the same lanes: lane group q
-// holds k = 32 s + 8 f(q) + (0..7) of k-step s, f = 0, 2, 1, 3.  Those are 8 consecutive fp8 weights, one ds_read_b64
-// (two per 16-byte DMA chunk; the weights are a ninth of the LDS reads), and the 16-byte token chunk 4 s + f(q) of a
+// holds k = 32 s + 8 f(q) + (0..7) of k-step s, f = 0, 2, 1, 3.  Those are 8 consecutive fp8 weights, one half of a
+// 16-byte part (read whole; the weights are a ninth of the LDS reads), and the 16-byte token chunk 4 s + f(q) of a
 // 64-k half.  128 token rows x 128 k would not fit LDS three times over next to the weights, so token rows travel in
 // halves of 64 k (128 rows x 128 bytes = 16 KiB) through three buffers of their own, one barrier per half, while the
 // weights keep their three buffers of 128 k: 96 + 48 KiB.  Per half-block a wave issues 2 weight DMA instructions (of
@@ -927,7 +927,7 @@ __device__ __forceinline__ void stream8x_tile(const GemmArgs& g, SBuf b0, SBuf b
     const int frow = lane & 15, q = lane >> 4;
     const int fq = ((q & 1) << 1) | (q >> 1);
     // weights: the 8 bytes at 32 s + 8 f(q) of the 64-byte half h of fragment row frow: 16-byte part 4 h + 2 s + f(q) / 2
-    const uint32_t w_rd = (uint32_t)(wave * 4096 + frow * 128 + (fq & 1) * 8), wkey = (uint32_t)wsw(frow);
+    const uint32_t w_rd = (uint32_t)(wave * 4096 + frow * 128), wkey = (uint32_t)wsw(frow);
     const uint32_t t_rd = (uint32_t)(frow * 128), tkey = (uint32_t)swz(frow);   // (group bases are multiples of 16 rows)
     f32x4 acc[TG][2];
 #pragma unroll
@@ -949,8 +949,13 @@ __device__ __forceinline__ void stream8x_tile(const GemmArgs& g, SBuf b0, SBuf b
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                wraw[s2][j] = *reinterpret_cast<const u32x2*>(wb.w + w_rd + j * 2048 + (((4 * h + 2 * s2 + (fq >> 1)) ^ wkey) << 4));
+            for (int j = 0; j < 2; ++j) {
+                // (the whole 16-byte part, of which this lane group uses one half and the group two further on the
+                // other: the two read the same address in the same LDS pass, a broadcast, where 8-byte reads of
+                // every other half collide -- SQ_LDS_BANK_CONFLICT was three times the LDS instruction cycles)
+                const u32x4 part = *reinterpret_cast<const u32x4*>(wb.w + w_rd + j * 2048 + (((4 * h + 2 * s2 + (fq >> 1)) ^ wkey) << 4));
+                wraw[s2][j] = (fq & 1) ? u32x2{part[2], part[3]} : u32x2{part[0], part[1]};
+            }
             const uint32_t coff = (uint32_t)(((4 * s2 + fq) ^ tkey) << 4);
 #pragma unroll
             for (int t = 0; t < TG; ++t) tf[s2][t] = *reinterpret_cast<const bf16x8*>(tb.t + t_rd + t * 16 * 128 + coff);
