@@ -373,13 +373,22 @@ def test_row_map_entry_outside_x_reads_zeros(h, I, n):
     assert (y_bad[bad].float().cpu().numpy() == 0).all()        # silu(0) * 0 through the down projection
 
 
-def test_gathered_rows_of_an_input_beyond_4_gib():
+@pytest.mark.parametrize("fp8", [False, True])
+def test_gathered_rows_of_an_input_beyond_4_gib(fp8):
     """Gathered rows are addressed with 32-bit byte offsets only while x is smaller than 4 GiB; a larger
-    x takes the one-workgroup-per-tile kernel with 64-bit addresses.  The rows used sit at both ends of x."""
+    x takes the one-workgroup-per-tile kernel with 64-bit addresses (with fp8 weights its register-staged body: the
+    weight streamers address rows through a 32-bit descriptor).  The rows used sit at both ends of x."""
     from moe_gen_amd import ops
     h, I, n = 2048, 256, 512
     x_rows = (1 << 32) // (h * 2) + 4096                          # 4 GiB + 16 MiB of bf16 rows
-    ws, ptrs = _one_expert(h, I, 43)
+    if fp8:
+        mats = make_experts(1, h, I, True, 43)[0]
+        dm = [tuple(t.cuda() for t in m) for m in mats]
+        ptrs = ops.expert_pointers([dm[0][0]], [dm[1][0]], [dm[2][0]], [dm[0][1]], [dm[1][1]], [dm[2][1]])
+        wg, wu, wd = (f32_of(m) for m in mats)
+    else:
+        ws, ptrs = _one_expert(h, I, 43)
+        wg, wu, wd = (O.bf16_to_f32(bits(w)) for w in ws)
     g = torch.Generator().manual_seed(44)
     rows = torch.randn(n, h, generator=g).to(torch.bfloat16)
     x = torch.zeros(x_rows, h, dtype=torch.bfloat16, device="cuda")
@@ -391,7 +400,6 @@ def test_gathered_rows_of_an_input_beyond_4_gib():
     y_ref = ops.grouped_swiglu(rows.cuda(), None, ptrs, off, n)   # the same rows, sorted: the persistent kernel
     torch.cuda.synchronize()
     del x
-    wg, wu, wd = (O.bf16_to_f32(bits(w)) for w in ws)
     ref32 = O.mlp_f32(O.bf16_to_f32(bits(rows)), wg, wu, wd)
     assert rel_max(O.bf16_to_f32(bits(y)), ref32) <= TOL
     assert rel_max(O.bf16_to_f32(bits(y_ref)), ref32) <= TOL
