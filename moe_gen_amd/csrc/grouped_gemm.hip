@@ -1100,6 +1100,172 @@ __device__ __forceinline__ int sum_over_experts(const GemmArgs& g, int tid, int*
     return tot;
 }
 
+// ---- bf16 weight streamer in the persistent kernel's summation order: tiles of up to 192 rows ----
+//
+// The fp8 streamers' way of moving data for bf16 weights: weights and token rows reach LDS by DMA in the persistent
+// kernel's layout of a 64-k stage (128-byte rows, chunk c of row r at c ^ swz(r)), and every matrix instruction gets
+// the k values the persistent kernel gives it, in the same lanes, so a row's bits do not depend on who computes it.
+// No staging registers and no LDS stores, so every operand of a stage can be requested up front.  Up to 64 rows the 8
+// waves split the tile's 256 weight rows and each multiplies all token rows; above, two sets of 4 waves take half of
+// the token groups each (4 + TG / 2 operand reads per k-step for 2 TG matrix instructions, where 8 x 1 waves need
+// 2 + TG for as many).  Three weight buffers of 32 KiB keep two stages of weights in flight; token rows (up to
+// 24 KiB per stage, out of L2) have two buffers and travel one stage ahead, issued first in a stage so that the wait
+// before the next stage's barrier leaves only the 4 weight instructions behind them in flight.
+// Weight row R of a stage (LDS row R, brought by wave R / 32): column n0 + R; gate and up: gate column n0 + R,
+// R < 128, up column n0 + R - 128 above.  k starts at stage 0 unless the kernel has the call to itself.
+template <int TG, bool SWIGLU, bool SHARED>   // TG: 16-row token groups multiplied (1 .. 12); SHARED: another tile reads these weights
+__device__ __forceinline__ void stream16_tile(const GemmArgs& g, uint8_t* w0, uint8_t* w1, uint8_t* w2, uint8_t* t0, uint8_t* t1,
+                                              int e, int row0, int row_end, int n_tile, bool rotate) {
+    constexpr int NBLK = SWIGLU ? 128 : 256;
+    constexpr int WM = TG >= 5 ? 2 : 1;           // sets of waves across the token groups
+    constexpr int TH = (TG + WM - 1) / WM;        // token groups per wave (an odd TG: the second set's last group is padding)
+    constexpr int NF = 2 * WM;                    // 16-row weight fragments per wave
+    constexpr int NDW = 4;                        // weight DMA instructions per wave and stage
+    constexpr int NDT = (2 * TG + 7) / 8;         // token DMA instructions per wave and stage (8 rows each; 64 rows per round of the waves)
+    static_assert(TG >= 1 && TG <= 12, "token rows staged");
+    const int tid = threadIdx.x, lane = tid & 63, wave = uni(tid >> 6);
+    const int wm = WM == 2 ? wave >> 2 : 0, wn = WM == 2 ? wave & 3 : wave;
+    const int n0 = n_tile * NBLK;
+    const int K = g.K, N = g.N;
+    const int nk = K / BK;
+    const int prot = rotate ? n_tile % nk : 0;
+
+    // ---- DMA coordinates: lane l supplies row +l/8 of an instruction's 8 rows and the 16 bytes that belong at physical chunk l%8 ----
+    const int lr = lane >> 3, pp = lane & 7;
+    uint32_t w_voff[NDW], t_voff[NDT];
+    const uint8_t* bmat = uni_ptr((SWIGLU && wave >= 4) ? g.b1[e] : g.b0[e]);
+#pragma unroll
+    for (int i = 0; i < NDW; ++i) {               // LDS rows 32 wave + 8 i + lr
+        const int R = 32 * wave + 8 * i + lr;
+        w_voff[i] = (uint32_t)min(n0 + (SWIGLU ? R & 127 : R), N - 1) * (uint32_t)(K * 2) + (uint32_t)((pp ^ swz(R)) << 4);
+    }
+    const uint8_t* a_base = reinterpret_cast<const uint8_t*>(g.a) + (g.row_map ? (size_t)0 : (size_t)row0 * K * 2);
+    const int a_records = g.row_map ? (int)(uint32_t)g.a_bytes : (row_end - row0) * K * 2;
+#pragma unroll
+    for (int i = 0; i < NDT; ++i) {               // token rows 64 i + 8 wave + lr; rows past the tile's last: zeros, no request
+        const int tr = 64 * i + 8 * wave + lr;
+        const int r = min(row0 + tr, row_end - 1);
+        const int src = g.row_map ? ((gptr_i32)(uintptr_t)g.row_map)[r] : r - row0;
+        t_voff[i] = (uint32_t)src * (uint32_t)(K * 2) + (uint32_t)((pp ^ swz(tr)) << 4);
+        if (row0 + tr >= row_end || (g.row_map && (unsigned)src >= (unsigned)g.a_rows)) t_voff[i] = 0xfffffff0u;
+    }
+    auto stage_off = [&](int kt_pipe) {           // byte offset of pipeline stage kt_pipe in a row (the last one again past the end)
+        int kt = min(kt_pipe, nk - 1) + prot;
+        kt = kt >= nk ? kt - nk : kt;
+        return (uint32_t)(kt * BK * 2);
+    };
+    auto dma_w = [&](int kt_pipe, uint8_t* wb, int i) __attribute__((always_inline)) {
+        const int live = uni(kt_pipe < nk ? -1 : 0);   // past the end: an empty descriptor, zeros without a request
+        const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)bmat, 0, live, 0x00020000);
+        // (non-temporal unless a neighbour on this XCD reads the same lines and should find them in its L2)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_u8)(wb + wave * 4096 + i * 1024), 16, w_voff[i], stage_off(kt_pipe), 0, SHARED ? 0 : 2);
+    };
+    auto dma_t = [&](int kt_pipe, uint8_t* tb, int i) __attribute__((always_inline)) {
+        const int live = uni(kt_pipe < nk ? -1 : 0);
+        const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)a_base, 0, live & a_records, 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_u8)(tb + (64 * i + 8 * wave) * ROW_B), 16, t_voff[i], stage_off(kt_pipe), 0, 0);
+    };
+
+    // ---- operand coordinates: fragment j of the wave is LDS rows wrow(j) .. + 15 ----
+    const int frow = lane & 15, q = lane >> 4;
+    const int fq = ((q & 1) << 1) | (q >> 1);
+    const uint32_t fkey = (uint32_t)swz(frow);
+    auto wrow = [&](int j) { return SWIGLU ? (j / WM) * 128 + 16 * WM * wn + 16 * (j % WM) : 32 * WM * wn + 16 * j; };
+    const uint32_t w_rd = (uint32_t)((wrow(0) + frow) * ROW_B), t_rd = (uint32_t)((16 * TH * wm + frow) * ROW_B);
+    f32x4 acc[TH][NF];
+#pragma unroll
+    for (int t = 0; t < TH; ++t)
+#pragma unroll
+        for (int j = 0; j < NF; ++j) acc[t][j] = f32x4{0};
+
+    // Stage kt is multiplied out of weight buffer kt % 3 and token buffer kt % 2.  Before it: this wave's DMA of its
+    // tokens (issued first in the stage before) and of everything older has landed, its LDS reads have returned, then
+    // everybody's (a bare s_barrier).  After the barrier every wave has left stage kt - 1: its token buffer takes
+    // stage kt + 1, its weight buffer stage kt + 2.
+    // Every operand of the stage is requested up front (4 + TG / 2 or 2 + TG reads per k-step): the matrix instructions
+    // then run behind the LDS pipeline instead of waiting out its latency one token group at a time.
+    bf16x8 wa0[NF], tf0[TH], wa1[NF], tf1[TH];
+    auto read_step = [&](const uint8_t* wb, const uint8_t* tb, int s, bf16x8 (&wa)[NF], bf16x8 (&tf)[TH]) __attribute__((always_inline)) {
+        const uint32_t coff = (uint32_t)(((4 * s + fq) ^ fkey) << 4);
+#pragma unroll
+        for (int j = 0; j < NF; ++j) wa[j] = *reinterpret_cast<const bf16x8*>(wb + w_rd + (wrow(j) - wrow(0)) * ROW_B + coff);
+#pragma unroll
+        for (int t = 0; t < TH; ++t) tf[t] = *reinterpret_cast<const bf16x8*>(tb + t_rd + t * 16 * ROW_B + coff);
+    };
+    // (with 2 of the 4 instructions of the weight DMA after the first token group)
+    auto mfma_step = [&](const bf16x8 (&wa)[NF], const bf16x8 (&tf)[TH], int kt_dma, uint8_t* w_refill, int i0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < TH; ++t) {
+#pragma unroll
+            for (int j = 0; j < NF; ++j) acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[j], tf[t], acc[t][j], 0, 0, 0);
+            if (t == 0) { dma_w(kt_dma, w_refill, i0); dma_w(kt_dma, w_refill, i0 + 1); }
+        }
+    };
+    auto stage = [&](int kt, const uint8_t* wb, const uint8_t* tb, uint8_t* w_refill, uint8_t* t_refill) __attribute__((always_inline)) {
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" :: "n"(NDW) : "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < NDT; ++i) dma_t(kt + 1, t_refill, i);
+        __builtin_amdgcn_sched_barrier(0);
+        read_step(wb, tb, 0, wa0, tf0);
+        read_step(wb, tb, 1, wa1, tf1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_step(wa0, tf0, kt + 2, w_refill, 0);
+        mfma_step(wa1, tf1, kt + 2, w_refill, 2);
+        __builtin_amdgcn_sched_barrier(0);      // (or the matrix instructions sink below the next stage's barrier, behind its reads)
+    };
+    // Prologue: the tokens of stage 0 between the weights of stages 0 and 1, so that the first wait (all but the 4
+    // youngest instructions) covers what stage 0 reads, as in the steady state.
+#pragma unroll
+    for (int i = 0; i < NDW; ++i) dma_w(0, w0, i);
+#pragma unroll
+    for (int i = 0; i < NDT; ++i) dma_t(0, t0, i);
+#pragma unroll
+    for (int i = 0; i < NDW; ++i) dma_w(1, w1, i);
+    // Six stages bring both rotations back to where they started: literal buffers in the loop body.
+    int kt = 0;
+    for (; kt + 6 <= nk; kt += 6) {
+        stage(kt, w0, t0, w2, t1);
+        stage(kt + 1, w1, t1, w0, t0);
+        stage(kt + 2, w2, t0, w1, t1);
+        stage(kt + 3, w0, t1, w2, t0);
+        stage(kt + 4, w1, t0, w0, t1);
+        stage(kt + 5, w2, t1, w1, t0);
+    }
+    if (kt < nk) stage(kt, w0, t0, w2, t1);
+    if (kt + 1 < nk) stage(kt + 1, w1, t1, w0, t0);
+    if (kt + 2 < nk) stage(kt + 2, w2, t0, w1, t1);
+    if (kt + 3 < nk) stage(kt + 3, w0, t1, w2, t0);
+    if (kt + 4 < nk) stage(kt + 4, w1, t0, w0, t1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no DMA may land in LDS after the workgroup has gone
+
+    // ---- epilogue: a lane holds 4 consecutive columns of one row per accumulator and stores them itself ----
+#pragma unroll
+    for (int t = 0; t < TH; ++t) {
+        const int r = row0 + 16 * (TH * wm + t) + frow;
+        if (r >= row_end) continue;
+#pragma unroll
+        for (int j = 0; j < (SWIGLU ? WM : NF); ++j) {
+            const int col = n0 + wrow(j) + 4 * q;
+            if (col < N) *reinterpret_cast<u32x2*>(g.c + (size_t)r * N + col) = epilogue_pack<SWIGLU>(acc[t][j], acc[t][SWIGLU ? WM + j : j]);
+        }
+    }
+}
+
+template <bool SWIGLU, bool SHARED>
+__device__ __forceinline__ void stream16(const GemmArgs& g, uint8_t* w0, uint8_t* w1, uint8_t* w2, uint8_t* t0, uint8_t* t1, int e,
+                                         int row0, int row_end, int n_tile, bool rotate) {
+    const int tg = (row_end - row0 + 15) >> 4;
+    switch (tg) {
+#define MOE_S16_CASE(n) case n: stream16_tile<n, SWIGLU, SHARED>(g, w0, w1, w2, t0, t1, e, row0, row_end, n_tile, rotate); break;
+    MOE_S16_CASE(1) MOE_S16_CASE(2) MOE_S16_CASE(3) MOE_S16_CASE(4) MOE_S16_CASE(5) MOE_S16_CASE(6)
+    MOE_S16_CASE(7) MOE_S16_CASE(8) MOE_S16_CASE(9) MOE_S16_CASE(10) MOE_S16_CASE(11)
+#undef MOE_S16_CASE
+    default: stream16_tile<12, SWIGLU, SHARED>(g, w0, w1, w2, t0, t1, e, row0, row_end, n_tile, rotate); break;
+    }
+}
+
 template <bool SWIGLU>
 __device__ __forceinline__ void stream8x(const GemmArgs& g, SBuf b0, SBuf b1, SBuf b2, int e, int row0, int row_end, int n_tile,
                                          bool rotate) {
@@ -1118,21 +1284,19 @@ __device__ __forceinline__ void stream8x(const GemmArgs& g, SBuf b0, SBuf b1, SB
 template <int WN, bool SWIGLU, bool W8>
 __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     constexpr int NT = 128 * WN;
-    // bf16 weights: two stages of the tallest tile (192 token rows + 256 weight rows).  fp8 weights: three weight
-    // arrays of 32 KiB and three token arrays of 16 KiB -- the buffers of the weight streamers, written by DMA, as
-    // separate objects so that a read of one waits for no DMA into another; gemm_tile's two stages (128 + 256 rows)
-    // are two pairs of them.
-    constexpr int WB = W8 ? S8_WBYTES : (192 + BN_ROWS) * ROW_B;
-    constexpr int TB = W8 ? 128 * ROW_B : 16;
-    __shared__ __attribute__((aligned(1024))) uint8_t lw0[WB];
-    __shared__ __attribute__((aligned(1024))) uint8_t lw1[WB];
-    __shared__ __attribute__((aligned(1024))) uint8_t lw2[W8 ? S8_WBYTES : 16];
+    // Three weight arrays of 32 KiB and token arrays of 16 KiB (fp8 weights: three, 128 rows) or 24 KiB (bf16: two,
+    // 192 rows) -- the buffers of the weight streamers, written by DMA, as separate objects so that a read of one
+    // waits for no DMA into another; gemm_tile's two stages (up to 128 token rows + 256 weight rows) are two pairs
+    // of them.
+    constexpr int TB = W8 ? 128 * ROW_B : 192 * ROW_B;
+    __shared__ __attribute__((aligned(1024))) uint8_t lw0[S8_WBYTES];
+    __shared__ __attribute__((aligned(1024))) uint8_t lw1[S8_WBYTES];
+    __shared__ __attribute__((aligned(1024))) uint8_t lw2[S8_WBYTES];
     __shared__ __attribute__((aligned(1024))) uint8_t lt0[TB];
     __shared__ __attribute__((aligned(1024))) uint8_t lt1[TB];
-    __shared__ __attribute__((aligned(1024))) uint8_t lt2[TB];
-    static_assert(S8_TROWS * 256 <= 128 * ROW_B, "token region of a streamer buffer");
-    auto stage = [&](int i, int mt) { return W8 ? Stage{i ? lt1 : lt0, i ? lw1 : lw0, i ? lw1 : lw0}
-                                                 : Stage{i ? lw1 : lw0, (i ? lw1 : lw0) + 64 * mt * ROW_B, i ? lw1 : lw0}; };
+    __shared__ __attribute__((aligned(1024))) uint8_t lt2[W8 ? TB : 16];
+    static_assert(S8_TROWS * 256 <= 128 * ROW_B && S8_WBYTES == BN_ROWS * ROW_B, "regions of a streamer buffer");
+    auto stage = [&](int i) { return Stage{i ? lt1 : lt0, i ? lw1 : lw0, i ? lw1 : lw0}; };
     const SBuf sb0{lw0, lt0}, sb1{lw1, lt1}, sb2{lw2, lt2};
     __shared__ int s_pref[MAX_E + 1];
     __shared__ int s_wtot[NT / 64];
@@ -1198,7 +1362,8 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
         const int r1 = min(uni(s_sel[4]), uni(s_sel[3]) + (m_tile + 1) * 256);
         if (r0 >= r1) return;
         if (W8 && s8_ok) stream8x<SWIGLU>(g, sb0, sb1, sb2, e, r0, r1, n_tile, false);
-        else gemm_tile<2, WN, SWIGLU, W8, false>(g, stage(0, 2), stage(1, 2), e, r0, r1, n_tile);
+        else if (s8_ok) stream16<SWIGLU, true>(g, lw0, lw1, lw2, lt0, lt1, e, r0, min(r1, r0 + 128), n_tile, false);
+        else gemm_tile<2, WN, SWIGLU, W8, false>(g, stage(0), stage(1), e, r0, r1, n_tile);
         return;
     }
     const int row_end = uni(s_sel[4]);
@@ -1221,13 +1386,35 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
         }
         return;
     }
-    if (row_end - first_row <= 64) gemm_tile<1, WN, SWIGLU, W8, true>(g, stage(0, 1), stage(1, 1), e, first_row, row_end, n_tile);
-    else if (row_end - first_row <= 128) gemm_tile<2, WN, SWIGLU, W8, true>(g, stage(0, 2), stage(1, 2), e, first_row, row_end, n_tile);
-    else if (!W8 && mt_e == 1) gemm_tile<3, WN, SWIGLU, W8, true>(g, stage(0, 3), stage(1, 3), e, first_row, row_end, n_tile);
-    else if (!W8 && row_end - first_row >= PAIR_LO && row_end - first_row <= PAIR_HI) {
-        const int r0 = first_row + m_tile * half_rows(row_end - first_row);
-        gemm_tile<3, WN, SWIGLU, W8, false>(g, stage(0, 3), stage(1, 3), e, r0, min(row_end, r0 + half_rows(row_end - first_row)), n_tile);
-    } else gemm_tile<2, WN, SWIGLU, W8, false>(g, stage(0, 2), stage(1, 2), e, first_row + m_tile * 128, row_end, n_tile);
+    // The rows of this workgroup: the expert's (one tile: up to 192 rows, 128 with fp8 weights), one half of an
+    // expert of PAIR_LO .. PAIR_HI rows (bf16), or a 128-row slice.
+    const int rows_e = row_end - first_row;
+    const bool pair = !W8 && rows_e >= PAIR_LO && rows_e <= PAIR_HI;
+    const int slice = pair ? half_rows(rows_e) : 128;
+    const int t0 = mt_e > 1 ? first_row + m_tile * slice : first_row, t1 = mt_e > 1 ? min(row_end, t0 + slice) : row_end;
+    if (!W8 && s8_ok) {
+        // bf16 weights: the weight streamer in the persistent kernel's order
+        if (mt_e == 1) stream16<SWIGLU, false>(g, lw0, lw1, lw2, lt0, lt1, e, t0, t1, n_tile, alone);
+        else stream16<SWIGLU, true>(g, lw0, lw1, lw2, lt0, lt1, e, t0, t1, n_tile, alone);
+        return;
+    }
+    // 4 GiB of gathered rows or more: the register-staged body, which addresses them with 64-bit offsets, 128 rows
+    // at a time
+    if (t1 - t0 <= 64) {
+        gemm_tile<1, WN, SWIGLU, W8, true>(g, stage(0), stage(1), e, t0, t1, n_tile);
+    } else if (mt_e == 1) {
+        gemm_tile<2, WN, SWIGLU, W8, true>(g, stage(0), stage(1), e, t0, min(t1, t0 + 128), n_tile);
+        if (t1 - t0 > 128) {
+            __syncthreads();
+            gemm_tile<2, WN, SWIGLU, W8, true>(g, stage(0), stage(1), e, t0 + 128, t1, n_tile);
+        }
+    } else {
+        gemm_tile<2, WN, SWIGLU, W8, false>(g, stage(0), stage(1), e, t0, min(t1, t0 + 128), n_tile);
+        if (t1 - t0 > 128) {
+            __syncthreads();
+            gemm_tile<2, WN, SWIGLU, W8, false>(g, stage(0), stage(1), e, t0 + 128, t1, n_tile);
+        }
+    }
 }
 
 // lane id produced where it is used: the compiler cannot hoist it (and everything derived from it)

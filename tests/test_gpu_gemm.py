@@ -257,6 +257,54 @@ def test_fp8_weight_streamer_rows_do_not_depend_on_the_tile(h, I):
     assert rel_max(O.bf16_to_f32(bits(ys[0])), ref) <= TOL
 
 
+@pytest.mark.parametrize("counts", [
+    [5, 16, 17, 32, 33, 64, 65, 80, 81, 96, 112, 128, 129, 144, 160, 176, 192] + [5] * 12,     # mean 59: one kernel
+    [192, 181, 170, 160, 150, 140, 130, 129, 257, 300, 384, 600, 5]])                          # mean 215: both kernels
+def test_bf16_weight_streamer_rows_do_not_depend_on_the_tile(counts):
+    """bf16 experts of up to 192 rows (and the halves of one of 257 ... 384) go through the bf16 weight streamer: one
+    body per number of 16-row groups, two wave layouts (up to 64 rows, above), weights and token rows by DMA.
+    Experts that share one set of weights and start with the same five rows: those rows come out bit-identical from
+    every body -- in the second list also from the persistent kernel (600 rows) and the halves of a pair --, against
+    the oracle within the layer bound, and the call gives the same bits every time it runs (a tile's buffers are
+    refilled while other waves still multiply; a missing wait shows as run-to-run differences)."""
+    from moe_gen_amd import ops
+    E, h, I = len(counts), 448, 640            # 7 / 10 stages of 64 k: 1 / 4 stages after the loop unrolled by six
+    print(f"bf16 streamer counts={counts}", flush=True)
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    n = int(offsets[-1])
+    g = torch.Generator().manual_seed(197)
+    x = torch.randn(n, h, generator=g).to(torch.bfloat16)
+    for e in range(1, E):
+        x[offsets[e]:offsets[e] + 5] = x[:5]
+    one = make_experts(1, h, I, False, 198)[0]
+    dm = [m.cuda() for m in one]
+    ptrs = ops.expert_pointers([dm[0]] * E, [dm[1]] * E, [dm[2]] * E)
+    off_d = torch.from_numpy(offsets).cuda()
+    xd = x.cuda()
+    ys = [ops.grouped_swiglu(xd, None, ptrs, off_d, n).clone() for _ in range(8)]
+    torch.cuda.synchronize()
+    for rep in range(1, 8):
+        assert torch.equal(ys[rep], ys[0]), f"call {rep} differs from call 0"
+    for e in range(1, E):
+        assert torch.equal(ys[0][offsets[e]:offsets[e] + 5], ys[0][:5]), f"expert {e} ({counts[e]} rows)"
+    wg, wu, wd = (f32_of(m) for m in one)
+    ref = O.mlp_f32(O.bf16_to_f32(bits(x)), wg, wu, wd)
+    assert rel_max(O.bf16_to_f32(bits(ys[0])), ref) <= TOL
+
+
+@pytest.mark.parametrize("h,I", [(448, 512), (576, 640), (704, 384), (384, 448)])   # 7/8, 9/10, 11/6, 6/7 stages of 64 k
+def test_bf16_weight_streamer_shapes_and_gather(h, I):
+    """The bf16 weight streamer on every token-group count and both sides of each boundary, with stage counts that
+    leave 0 ... 5 stages after its loop unrolled by six, rows gathered through row_map, and last N tiles that are
+    ragged (down projection: h = 448, 576, 704 of 256 columns; gate/up: I = 448 of 128)."""
+    counts = [16, 17, 32, 33, 48, 49, 64, 65, 80, 81, 96, 97, 112, 113, 128, 129, 144, 145, 160, 161, 176, 177, 192,
+              1, 0, 15, 31, 47, 63] + [2] * 20
+    print(f"bf16 streamer shapes h={h} I={I} counts={counts}", flush=True)
+    y, ref32, refr = run_case(len(counts), h, I, counts, False, seed=161, use_row_map=True)
+    assert np.isfinite(y).all()
+    assert rel_max(y, ref32) <= TOL and rel_max(y, refr) <= TOL
+
+
 @pytest.mark.parametrize("h,I", [(512, 640), (640, 896), (896, 512)])      # 4 / 5 / 7 blocks of 128 k (gate/up), 5 / 7 / 4 (down)
 def test_fp8_weight_streamer_shapes_and_gather(h, I):
     """The fp8 weight streamer on every token-group count and both sides of each boundary, with block counts that
@@ -269,17 +317,22 @@ def test_fp8_weight_streamer_shapes_and_gather(h, I):
     assert rel_max(y, ref32) <= TOL and rel_max(y, refr) <= TOL
 
 
-def test_fp8_weight_streamer_row_outside_x_reads_zeros():
-    """A row_map entry outside x is a row of zeros for the streamer too (its token DMA goes through a bounds-checked
-    descriptor; such a row and the rows past an expert's last cost no memory request), and its neighbours are
-    untouched: the other rows' bits equal those of a call with valid entries only."""
+@pytest.mark.parametrize("fp8", [False, True])
+def test_weight_streamer_row_outside_x_reads_zeros(fp8):
+    """A row_map entry outside x is a row of zeros for the weight streamers too (their token DMA goes through a
+    bounds-checked descriptor; such a row and the rows past an expert's last cost no memory request), and its
+    neighbours are untouched: the other rows' bits equal those of a call with valid entries only."""
     from moe_gen_amd import ops
     E, h, I, per = 6, 512, 384, 20
     n = E * per
-    mats = make_experts(E, h, I, True, 5)
-    dm = [[tuple(t.cuda() for t in m) for m in one] for one in mats]
-    ptrs = ops.expert_pointers([o[0][0] for o in dm], [o[1][0] for o in dm], [o[2][0] for o in dm],
-                               [o[0][1] for o in dm], [o[1][1] for o in dm], [o[2][1] for o in dm])
+    mats = make_experts(E, h, I, fp8, 5)
+    if fp8:
+        dm = [[tuple(t.cuda() for t in m) for m in one] for one in mats]
+        ptrs = ops.expert_pointers([o[0][0] for o in dm], [o[1][0] for o in dm], [o[2][0] for o in dm],
+                                   [o[0][1] for o in dm], [o[1][1] for o in dm], [o[2][1] for o in dm])
+    else:
+        dm = [[m.cuda() for m in one] for one in mats]
+        ptrs = ops.expert_pointers([o[0] for o in dm], [o[1] for o in dm], [o[2] for o in dm])
     x = torch.randn(n, h, generator=torch.Generator().manual_seed(6)).to(torch.bfloat16).cuda()
     off = torch.arange(0, n + 1, per, dtype=torch.int32).cuda()
     rm = torch.arange(n, dtype=torch.int32)
