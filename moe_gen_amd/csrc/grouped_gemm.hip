@@ -101,6 +101,19 @@ struct GemmArgs {
 // two rows per cycle), so 16-byte operand reads by 32 consecutive rows never collide.
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
+// Stage at which a tile of N tile n_tile starts its walk over k.  Workgroups that run side by side mostly differ in
+// their N tile; started at the same stage, their requests in flight would share the low address bits (rows of the weight
+// matrices are K elements apart) and crowd the same memory channels: with the start spread over the stages a launch
+// that streams weights gains about a tenth (Mixtral-8x22B shapes, 8 experts x 16 ... 120 rows: 6.1 -> 6.8, 5.4 -> 6.1
+// TB/s; 128 / 160 / 192 rows next to the persistent kernel: gate/up 0.63 / 0.64 / 0.66 -> 0.55 / 0.58 / 0.62 ms).
+// bf16 weights: every path of both kernels uses this rule, so which kernel or tile computes a row does not change the
+// order its products are added in (the persistent kernel itself runs within 0.5 % either way).  fp8 weights (a scale
+// per 128 k: pairs of stages stay together): only in calls that the one-workgroup-per-tile kernel serves alone; the
+// persistent kernel loses 1.6 % of the DeepSeek-V3 step to a rotated walk, so calls that launch it start every tile
+// at stage 0, in both kernels.
+template <bool W8>
+__device__ __forceinline__ int k_rotation(int n_tile, int nk) { return (W8 ? 2 * n_tile : n_tile) % nk; }
+
 // global-address-space views: expert pointers come out of a pointer table in memory, and
 // without the address space the compiler must emit flat loads, whose completion is tracked
 // by the same counter as the LDS reads of the MFMA operands
@@ -312,19 +325,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, Stage st0, Stage st
     const int n0 = n_tile * NBLK;
     const int K = g.K, N = g.N;
     const int nk = K / BK;
-    // These tiles mostly stream weights, and neighbouring workgroups start together: were they all to walk k from 0,
-    // every request in flight on the chip would carry the same low address bits (rows are K elements apart) and
-    // crowd a few memory channels.  N tile t walks k from stage t instead (mod nk; a dot product does not care
-    // where it starts, and a column's order depends on nothing but its position, whatever the tile height):
-    // Mixtral-8x22B, 256 tokens, down projection 0.302 -> 0.273 ms, gate/up 0.640 -> 0.620 ms.
-    // fp8 weights under tiles below 256 rows are fetched 128 k at a time (see PAIR8 below): pairs of stages stay
-    // together, so fp8 tiles start at stage 2 t.  Only where this kernel has the call to itself: in a call that also
-    // launches the persistent kernel, which of the two computes a row depends on its expert's count or (fp8) on the
-    // row's position among its expert's rows, so both add in the same order, the persistent kernel's, from stage 0
-    // (DeepSeek-V2-Lite, 4096 tokens: 6 us of the 0.36 ms gate/up call).
+    // (fp8 weights under tiles below 256 rows are fetched 128 k at a time, see PAIR8 below: k_rotation keeps their
+    // pairs of stages together)
     constexpr bool PAIR8 = W8;
-    const bool alone = g.cold_max == 0x7fffffff;
-    const int rot = !alone ? 0 : W8 ? (2 * n_tile) % nk : n_tile % nk;
+    const int rot = (W8 && g.cold_max != 0x7fffffff) ? 0 : k_rotation<W8>(n_tile, nk);
     auto stage_at = [&](int kt) { const int kp = kt + rot; return kp >= nk ? kp - nk : kp; };
 
     // ---- per-thread load coordinates ----
@@ -864,7 +868,7 @@ __device__ __forceinline__ void stream8x_tile(const GemmArgs& g, SBuf b0, SBuf b
     const int n0 = n_tile * NBLK;
     const int K = g.K, N = g.N;
     const int npair = K >> 7;
-    const int prot = rotate ? n_tile % npair : 0;
+    const int prot = rotate ? n_tile % npair : 0;             // k_rotation in blocks of 128 k
 
     // ---- DMA coordinates ----
     // weights, instruction i (0..3): rows 8 i + lane / 8 of the wave's 32 (fragment i / 2, fragment row 8 (i & 1) + lane / 8);
@@ -1115,7 +1119,7 @@ __device__ __forceinline__ int sum_over_experts(const GemmArgs& g, int tid, int*
 // R < 128, up column n0 + R - 128 above.  k starts at stage 0 unless the kernel has the call to itself.
 template <int TG, bool SWIGLU, bool SHARED>   // TG: 16-row token groups multiplied (1 .. 12); SHARED: another tile reads these weights
 __device__ __forceinline__ void stream16_tile(const GemmArgs& g, uint8_t* w0, uint8_t* w1, uint8_t* w2, uint8_t* t0, uint8_t* t1,
-                                              int e, int row0, int row_end, int n_tile, bool rotate) {
+                                              int e, int row0, int row_end, int n_tile) {
     constexpr int NBLK = SWIGLU ? 128 : 256;
     constexpr int WM = TG >= 5 ? 2 : 1;           // sets of waves across the token groups
     constexpr int TH = (TG + WM - 1) / WM;        // token groups per wave (an odd TG: the second set's last group is padding)
@@ -1128,7 +1132,7 @@ __device__ __forceinline__ void stream16_tile(const GemmArgs& g, uint8_t* w0, ui
     const int n0 = n_tile * NBLK;
     const int K = g.K, N = g.N;
     const int nk = K / BK;
-    const int prot = rotate ? n_tile % nk : 0;
+    const int prot = k_rotation<false>(n_tile, nk);
 
     // ---- DMA coordinates: lane l supplies row +l/8 of an instruction's 8 rows and the 16 bytes that belong at physical chunk l%8 ----
     const int lr = lane >> 3, pp = lane & 7;
@@ -1255,14 +1259,14 @@ __device__ __forceinline__ void stream16_tile(const GemmArgs& g, uint8_t* w0, ui
 
 template <bool SWIGLU, bool SHARED>
 __device__ __forceinline__ void stream16(const GemmArgs& g, uint8_t* w0, uint8_t* w1, uint8_t* w2, uint8_t* t0, uint8_t* t1, int e,
-                                         int row0, int row_end, int n_tile, bool rotate) {
+                                         int row0, int row_end, int n_tile) {
     const int tg = (row_end - row0 + 15) >> 4;
     switch (tg) {
-#define MOE_S16_CASE(n) case n: stream16_tile<n, SWIGLU, SHARED>(g, w0, w1, w2, t0, t1, e, row0, row_end, n_tile, rotate); break;
+#define MOE_S16_CASE(n) case n: stream16_tile<n, SWIGLU, SHARED>(g, w0, w1, w2, t0, t1, e, row0, row_end, n_tile); break;
     MOE_S16_CASE(1) MOE_S16_CASE(2) MOE_S16_CASE(3) MOE_S16_CASE(4) MOE_S16_CASE(5) MOE_S16_CASE(6)
     MOE_S16_CASE(7) MOE_S16_CASE(8) MOE_S16_CASE(9) MOE_S16_CASE(10) MOE_S16_CASE(11)
 #undef MOE_S16_CASE
-    default: stream16_tile<12, SWIGLU, SHARED>(g, w0, w1, w2, t0, t1, e, row0, row_end, n_tile, rotate); break;
+    default: stream16_tile<12, SWIGLU, SHARED>(g, w0, w1, w2, t0, t1, e, row0, row_end, n_tile); break;
     }
 }
 
@@ -1362,7 +1366,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
         const int r1 = min(uni(s_sel[4]), uni(s_sel[3]) + (m_tile + 1) * 256);
         if (r0 >= r1) return;
         if (W8 && s8_ok) stream8x<SWIGLU>(g, sb0, sb1, sb2, e, r0, r1, n_tile, false);
-        else if (s8_ok) stream16<SWIGLU, true>(g, lw0, lw1, lw2, lt0, lt1, e, r0, min(r1, r0 + 128), n_tile, false);
+        else if (s8_ok) stream16<SWIGLU, true>(g, lw0, lw1, lw2, lt0, lt1, e, r0, min(r1, r0 + 128), n_tile);
         else gemm_tile<2, WN, SWIGLU, W8, false>(g, stage(0), stage(1), e, r0, r1, n_tile);
         return;
     }
@@ -1394,8 +1398,8 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     const int t0 = mt_e > 1 ? first_row + m_tile * slice : first_row, t1 = mt_e > 1 ? min(row_end, t0 + slice) : row_end;
     if (!W8 && s8_ok) {
         // bf16 weights: the weight streamer in the persistent kernel's order
-        if (mt_e == 1) stream16<SWIGLU, false>(g, lw0, lw1, lw2, lt0, lt1, e, t0, t1, n_tile, alone);
-        else stream16<SWIGLU, true>(g, lw0, lw1, lw2, lt0, lt1, e, t0, t1, n_tile, alone);
+        if (mt_e == 1) stream16<SWIGLU, false>(g, lw0, lw1, lw2, lt0, lt1, e, t0, t1, n_tile);
+        else stream16<SWIGLU, true>(g, lw0, lw1, lw2, lt0, lt1, e, t0, t1, n_tile);
         return;
     }
     // 4 GiB of gathered rows or more: the register-staged body, which addresses them with 64-bit offsets, 128 rows
@@ -1513,6 +1517,11 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
     gptr_f32 sc0 = nullptr, sc1 = nullptr;
     int row0 = 0, row_end = 0, n0 = 0;
     int cur_e = 0;
+    // bf16 weights: k starts at another stage for every N tile (k_rotation); stage_of is the stage that pipeline step
+    // kt fetches.  The rotation is adopted with the tile's DMA coordinates.
+    const int nk = K / BK;
+    int rot = 0, rot_n = 0;
+    auto stage_of = [&](int kt, int r) { const int kp = kt + r; return kp >= nk ? kp - nk : kp; };
     auto setup = [&](int v) {
         const int l = fresh_lane();
         const int t = wave_s * 64 + l;
@@ -1526,6 +1535,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
         row0 = uni(s_off[e]) + m_tile * BM;
         row_end = uni(s_off[e + 1]);
         n0 = n_tile * NBLK;
+        rot_n = W8 ? 0 : k_rotation<false>(n_tile, nk);
         // DMA instruction i of this wave fills rows 32*wave + 8*i .. +7 of a stage: lane l supplies row +l/8 and
         // the 16 bytes that belong at physical chunk l%8, i.e. logical chunk (l%8) ^ swz(row)
         const int lr = l >> 3, pc = l & 7;
@@ -1570,16 +1580,17 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
         for (int i = 0; i < ND; ++i) { a_voff[i] = a_voff_n[i]; if (!W8) b_voff[i] = b_voff_n[i]; }
         if (!W8) bm_cur = bm_next;
         a_base = a_base_n;
+        rot = rot_n;
     };
     auto dma_a = [&](uint8_t* stA, int kt, int i) {
         const __amdgpu_buffer_rsrc_t rsrcA = __builtin_amdgcn_make_buffer_rsrc((void*)a_base, 0, a_records, 0x00020000);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lds_u8)(stA + (32 * wave_s + 8 * i) * ROW_B), 16, a_voff[i],
-                                                 (uint32_t)(kt * BK * 2), 0, 0);
+                                                 (uint32_t)((W8 ? kt : stage_of(kt, rot)) * BK * 2), 0, 0);
     };
     auto dma_b = [&](uint8_t* stB, int kt, int i) {
         const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)bm_cur, 0, -1, 0x00020000);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_u8)(stB + (32 * wave_s + 8 * i) * ROW_B), 16, b_voff[i],
-                                                 (uint32_t)(kt * BK * 2), 0, 0);
+                                                 (uint32_t)((W8 ? kt : stage_of(kt, rot)) * BK * 2), 0, 0);
     };
     // fp8 weight path (registers): thread t owns row t/4 (+128 i), chunks 2q, 2q+1 of the bf16 row
     const int brow = tid >> 2;
@@ -1660,7 +1671,6 @@ __global__ __launch_bounds__(512) void grouped_gemm_persistent_kernel(GemmArgs g
                 acc[q * TQ + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wfr[s][j], tq[u & 1][i], acc[q * TQ + i][j], 0, 0, 0);
             }
     };
-    const int nk = K / BK;
     constexpr int WPS = TN / NP;
     // iteration kt multiplies stage par; the DMA brings k-stage ka (of the tile whose coordinates are current) into
     // the other token stage (and weight stage, bf16); fp8 converts the weight registers (k-stage kt+1) into the other
