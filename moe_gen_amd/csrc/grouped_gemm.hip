@@ -26,20 +26,21 @@
 //  * grouped_gemm_kernel (experts of up to 192 rows, 128 with fp8 weights, and with fp8 weights what an
 //    expert's full 256-row tiles leave over; work that mostly streams weights): one
 //    workgroup per tile, grid = upper bound on the tile count, surplus workgroups exit at once;
-//    the tile height (64, 128 or 192 rows) follows the expert, groups of 4 tiles go round-robin
-//    to the XCDs.
+//    the tile height (16 ... 192 rows in steps of 16) follows the expert, groups of 4 tiles go round-robin
+//    to the XCDs.  Its tiles run through the weight streamers (stream16_tile, stream8x_tile, stream8_tile):
+//    weights AND token rows reach LDS by DMA, three weight buffers, one barrier per stage.
 //
-// Workgroup = 8 waves (2 along M, 4 along N), two per SIMD.  Per wave 2, 4, 6 or 8 x 4 MFMA tiles
-// of 16x16 (v_mfma_f32_16x16x32_bf16), i.e. up to 128x64 outputs and 128 fp32 accumulators.  On
-// real (non-zero) data this chip is power-limited under MFMA load; the 16x16x32 shape moves a
-// third less accumulator data per flop than 32x32x16 and sustains ~13 % more (1.95 vs 1.73
-// PFLOP/s in a registers-only loop with random operands), which is worth ~6 % here.
-// K advances 64 at a time through two LDS stages; rows are 128 bytes with a 16-byte-chunk
-// XOR swizzle so that both the 16-byte stores and the 16-byte MFMA operand reads are
-// bank-conflict free.  Global loads for tile k+2 are in flight while tile k is multiplied
-// and tile k+1 is written to LDS; every wave interleaves its share of that data movement with
-// its MFMAs, one piece per group of MFMAs, between the one barrier per k-stage.  The persistent
-// kernel brings token rows and bf16 weights into LDS by DMA instead (buffer_load ... lds).
+// Workgroup = 8 waves, two per SIMD.  v_mfma_f32_16x16x32_bf16 throughout: on real (non-zero) data this
+// chip is power-limited under MFMA load; the 16x16x32 shape moves a third less accumulator data per flop
+// than 32x32x16 and sustains ~13 % more (1.95 vs 1.73 PFLOP/s in a registers-only loop with random
+// operands), which is worth ~6 % here.  The persistent kernel's waves are 2 along M x 4 along N, 8 x 4 MFMA
+// tiles each (128x64 outputs, 128 fp32 accumulators).  K advances 64 at a time through two LDS stages; rows
+// are 128 bytes with a 16-byte-chunk XOR swizzle so that both the 16-byte stores and the 16-byte MFMA
+// operand reads are bank-conflict free.  Token rows and bf16 weights come into LDS by DMA
+// (buffer_load ... lds); fp8 weights of the persistent kernel go through registers, converted on the way,
+// two k-stages ahead, every wave interleaving its share of that with its MFMAs, one piece per group of
+// MFMAs, between the one barrier per k-stage.  gemm_tile, the register-staged body of the other kernel,
+// remains for calls that gather from 4 GiB of rows or more (the DMA paths address them with 32 bits).
 //
 // The MFMA is issued with the WEIGHT fragment as srcA and the TOKEN fragment as srcB, so
 // a lane ends up holding 4 consecutive output columns of one token row per accumulator;

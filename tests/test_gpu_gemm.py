@@ -292,6 +292,32 @@ def test_bf16_weight_streamer_rows_do_not_depend_on_the_tile(counts):
     assert rel_max(O.bf16_to_f32(bits(ys[0])), ref) <= TOL
 
 
+def test_bf16_rows_do_not_depend_on_the_call():
+    """With bf16 weights every path of both kernels adds a column's products in one order, in every call: the same 40
+    rows come out bit-identical from a call that the one-workgroup-per-tile kernel serves alone (one expert of 40
+    rows) and from a call that launches both kernels, where they open an expert of 600 rows (persistent kernel), one
+    of 150 (a single tile) and one of 300 (the first of two tiles side by side)."""
+    from moe_gen_amd import ops
+    h, I, r = 512, 768, 40
+    g = torch.Generator().manual_seed(211)
+    rows = torch.randn(r, h, generator=g).to(torch.bfloat16)
+    one = make_experts(1, h, I, False, 212)[0]
+    dm = [m.cuda() for m in one]
+    small = ops.grouped_swiglu(rows.cuda(), None, ops.expert_pointers([dm[0]], [dm[1]], [dm[2]]),
+                               torch.tensor([0, r], dtype=torch.int32).cuda(), r)
+    counts = [600, 150, 300]
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    n = int(offsets[-1])
+    x = torch.randn(n, h, generator=g).to(torch.bfloat16)
+    for e in range(3):
+        x[offsets[e]:offsets[e] + r] = rows
+    big = ops.grouped_swiglu(x.cuda(), None, ops.expert_pointers([dm[0]] * 3, [dm[1]] * 3, [dm[2]] * 3),
+                             torch.from_numpy(offsets).cuda(), n)
+    torch.cuda.synchronize()
+    for e in range(3):
+        assert torch.equal(big[offsets[e]:offsets[e] + r], small), f"expert of {counts[e]} rows"
+
+
 @pytest.mark.parametrize("h,I", [(448, 512), (576, 640), (704, 384), (384, 448)])   # 7/8, 9/10, 11/6, 6/7 stages of 64 k
 def test_bf16_weight_streamer_shapes_and_gather(h, I):
     """The bf16 weight streamer on every token-group count and both sides of each boundary, with stage counts that
