@@ -370,6 +370,7 @@ def run_workload(name: str, args, with_cpu: bool):
     dev = "cuda:0"
     blk = synthetic.build_block(w, device=dev, gen_device=dev)
     blk.fused_gather = not args.materialize
+    blk.join_shared = not args.no_join_shared
     x = synthetic.hidden_states(w, dev)
     torch.cuda.synchronize()
     for _ in range(args.warmup):
@@ -413,7 +414,10 @@ def run_workload(name: str, args, with_cpu: bool):
     # dominant kernel: the fused gate/up SwiGLU GEMM.  With shared experts it is launched twice per
     # step (routed experts, shared expert; same kernel, different row counts): algorithmic FLOP per
     # launch and average launch duration are both averages over those launches.
-    gu_flop = [4.0 * w.n * w.k * w.h * w.I]
+    # (At small token counts the block runs a single shared expert as one more group of the routed call: then the
+    # "routed" launches carry its rows too and there are no launches of its own.)
+    joined = w.S > 0 and "shared_gate_up" not in st
+    gu_flop = [4.0 * w.n * w.k * w.h * w.I + (4.0 * w.n * w.h * w.S * w.I if joined else 0.0)]
     gu_ms = [st["routed_gate_up"]]
     if "shared_gate_up" in st:
         gu_flop.append(4.0 * w.n * w.h * w.S * w.I)
@@ -444,8 +448,9 @@ def run_workload(name: str, args, with_cpu: bool):
         if cal:
             keys = ("vendor_dense_tflops", "own_dense_bf16_tflops", "vendor_dense_down_tflops", "own_dense_bf16_down_tflops")
             mean = {k: sum(c[k] for c in cal) / len(cal) for k in keys}
-            routed_gu = 4.0 * w.n * w.k * w.h * w.I / (st["routed_gate_up"] * 1e-3) / 1e12
-            routed_dn = 2.0 * w.n * w.k * w.h * w.I / (st["routed_down"] * 1e-3) / 1e12
+            rows = w.n * w.k + (w.n * w.S if joined else 0)
+            routed_gu = 4.0 * rows * w.h * w.I / (st["routed_gate_up"] * 1e-3) / 1e12
+            routed_dn = 2.0 * rows * w.h * w.I / (st["routed_down"] * 1e-3) / 1e12
             roofline["calibration"] = {**mean, "before_timed_passes": {k: cal[0][k] for k in keys},
                                        "after_timed_passes": {k: cal[1][k] for k in keys}, "shape": cal[0]["shape"],
                                        "reps": cal[0]["reps"],
@@ -461,6 +466,8 @@ def run_workload(name: str, args, with_cpu: bool):
         # few rows per expert: the launch streams every expert's gate and up matrix once and is bound by HBM.
         # Algorithmic bytes per launch: both matrices of every expert, the gathered token rows, the activations out.
         gu_bytes = 2.0 * w.E * w.h * w.I * (1 if w.fp8 else 2) + 2.0 * w.n * w.k * (w.h + w.I)
+        if joined:                                   # (+ the shared expert's matrices, rows and activations)
+            gu_bytes += 2.0 * w.S * w.h * w.I * (1 if w.fp8 else 2) + 2.0 * w.n * (w.h + w.S * w.I)
         gbps = gu_bytes / (st["routed_gate_up"] * 1e-3) / 1e9
         roofline = {"bound": "hbm",
                     "kernel": f"grouped_gemm_kernel<WN=4,SWIGLU=true,W8={w8}> (gate/up + SiLU*mul, one workgroup per tile)",
@@ -605,6 +612,8 @@ def main():
     ap.add_argument("--all-workloads", action="store_true", help="(default) every synthetic workload in the one JSON line")
     ap.add_argument("--headline-only", action="store_true", help="only the workload named by --workload")
     ap.add_argument("--tokens", type=int, default=0, help="override the token count (parity/debug only)")
+    ap.add_argument("--no-join-shared", action="store_true", help="keep a single shared expert in a grouped call of "
+                    "its own at every token count (by default it joins the routed call at small batches)")
     ap.add_argument("--materialize", action="store_true", help="gather rows into a sorted copy instead of "
                     "reading them through the row map inside the GEMM")
     ap.add_argument("--no-cpu-baseline", action="store_true")

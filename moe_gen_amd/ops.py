@@ -99,10 +99,13 @@ class Dispatch(NamedTuple):
     row_map: torch.Tensor | None     # int32 [n*k] = perm // k (only when asked for)
 
 
-def dispatch(topk_idx: torch.Tensor, n_experts: int, x: torch.Tensor | None = None, want_row_map: bool = False):
+def dispatch(topk_idx: torch.Tensor, n_experts: int, x: torch.Tensor | None = None, want_row_map: bool = False,
+             out_row_map: torch.Tensor | None = None):
     """topk_idx int32 [n,k] -> Dispatch(counts [E], offsets [E+1], perm [n*k], pos [n*k], xs, row_map):
     if x bf16 [n,h] is given, xs holds the gathered rows [n*k,h]; with want_row_map, row_map[r] is
-    the token row behind sorted row r (the grouped GEMM gathers through it)."""
+    the token row behind sorted row r (the grouped GEMM gathers through it).
+    out_row_map: an int32 device buffer of at least n*k entries to write the row map into (its first n*k entries; a
+    caller that adds groups of its own to the grouped call passes a slice of a longer map); it is returned as given."""
     _need(topk_idx, torch.int32, "topk_idx")
     n, k = topk_idx.shape
     dev = topk_idx.device
@@ -110,7 +113,13 @@ def dispatch(topk_idx: torch.Tensor, n_experts: int, x: torch.Tensor | None = No
     offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=dev)
     perm = torch.empty(n * k, dtype=torch.int32, device=dev)
     pos = torch.empty(n * k, dtype=torch.int32, device=dev)
-    row_map = torch.empty(n * k, dtype=torch.int32, device=dev) if want_row_map else None
+    if out_row_map is not None:
+        _need(out_row_map, torch.int32, "out_row_map")
+        if out_row_map.numel() < n * k:
+            raise ValueError(f"out_row_map holds {out_row_map.numel()} entries, {n * k} needed")
+        want_row_map = True
+    row_map = out_row_map if out_row_map is not None else (
+        torch.empty(n * k, dtype=torch.int32, device=dev) if want_row_map else None)
     xs, h = None, 0
     if x is not None:
         _need(x, torch.bfloat16, "x")

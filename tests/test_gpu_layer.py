@@ -158,3 +158,36 @@ def test_block_forward_can_be_captured_in_a_graph(name):
     graph.replay()
     torch.cuda.synchronize()
     assert torch.equal(y_static, y2), "replay on a new input differs from the eager forward"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fp8", [False, True])
+def test_single_shared_expert_joins_the_routed_call_at_small_batches(fp8):
+    """A DeepSeek-V3-shaped block (one shared expert of the routed experts' shape) under a small batch runs the shared
+    expert as one more group of the routed experts' grouped call.  The stage timer then shows no launches of its own,
+    and with bf16 weights the output equals, bit for bit, what the two separate calls give (every bf16 path adds in
+    one order); with fp8 weights the two agree within the layer bound, since a call that the one-workgroup-per-tile
+    kernel serves alone adds in another order than the persistent kernel.  (test_block_vs_oracle holds the joined
+    path to the oracle: its DeepSeek-V3 cases are small batches.)"""
+    from moe_gen_amd import synthetic
+    from moe_gen_amd.block import StageTimer
+    w = synthetic.WORKLOADS["deepseek_v3_w8a16"].scaled(n=384, h=512, I=256, seq=64, fp8=fp8)
+    blk = synthetic.build_block(w, device="cuda:0", gen_device="cpu")
+    x = synthetic.hidden_states(w, "cpu").to("cuda:0")
+    blk.stage_timer = StageTimer()
+    joined = blk(x)
+    torch.cuda.synchronize()
+    keys = set(blk.stage_timer.totals_ms())
+    blk.stage_timer = StageTimer()
+    blk.join_shared = False
+    apart = blk(x)
+    torch.cuda.synchronize()
+    keys_apart = set(blk.stage_timer.totals_ms())
+    blk.stage_timer = None
+    assert "shared_gate_up" not in keys and "routed_gate_up" in keys
+    assert "shared_gate_up" in keys_apart
+    a, b = joined.float(), apart.float()
+    if fp8:
+        assert (a - b).abs().max().item() <= 2e-2 * b.abs().max().item()
+    else:
+        assert torch.equal(joined, apart)
