@@ -484,6 +484,37 @@ def test_gathered_rows_of_an_input_beyond_4_gib(fp8):
     assert rel_max(O.bf16_to_f32(bits(y_ref)), ref32) <= TOL
 
 
+def test_gathered_rows_beyond_4_gib_at_every_tile_kind_bf16():
+    """The register-staged body behind the bf16 weight streamer (4 GiB of gathered rows or more) takes what the
+    streamer takes: single tiles of up to 192 rows (above 128 as two passes of 128 rows), the halves of an expert of
+    257 to 384 rows, 128-row slices.  Experts that share one set of weights, rows gathered from both ends of a 4 GiB
+    x: every row equals, bit for bit, what the same rows give sorted and through the streamer (one order of
+    summation for every bf16 path)."""
+    from moe_gen_amd import ops
+    h, I = 2048, 256
+    counts = [150, 192, 300, 40, 129, 70, 384, 500]
+    E, n = len(counts), sum(counts)
+    x_rows = (1 << 32) // (h * 2) + 4096                          # 4 GiB + 16 MiB of bf16 rows
+    ws, _ = _one_expert(h, I, 47)
+    dw = [w.cuda() for w in ws]
+    ptrs = ops.expert_pointers([dw[0]] * E, [dw[1]] * E, [dw[2]] * E)
+    g = torch.Generator().manual_seed(48)
+    rows = torch.randn(n, h, generator=g).to(torch.bfloat16)
+    x = torch.zeros(x_rows, h, dtype=torch.bfloat16, device="cuda")
+    where = torch.cat([torch.arange(n // 2), torch.arange(x_rows - (n - n // 2), x_rows)]).to(torch.int32)
+    where = where[torch.randperm(n, generator=g)]
+    x[where.long().cuda()] = rows.cuda()
+    off = torch.tensor(np.concatenate([[0], np.cumsum(counts)]), dtype=torch.int32, device="cuda")
+    print(f"4 GiB gather, bf16, counts={counts}", flush=True)
+    y = ops.grouped_swiglu(x, where.cuda(), ptrs, off, n)
+    y_ref = ops.grouped_swiglu(rows.cuda(), None, ptrs, off, n)
+    torch.cuda.synchronize()
+    del x
+    wg, wu, wd = (O.bf16_to_f32(bits(w)) for w in ws)
+    assert rel_max(O.bf16_to_f32(bits(y_ref)), O.mlp_f32(O.bf16_to_f32(bits(rows)), wg, wu, wd)) <= TOL
+    assert torch.equal(y, y_ref)
+
+
 @pytest.mark.parametrize("fp8", [False, True])
 def test_expert_sub_range_through_the_persistent_kernel(fp8):
     """A call on experts [1, 3) of four with absolute row offsets (weights handed out in waves): the rows
