@@ -23,11 +23,11 @@
 //    ids are dealt to the 8 XCDs one by one by the hardware; the tiles of a group share their
 //    A and B panels through that XCD's L2), and a workgroup's k pipeline runs on from one of
 //    its tiles into the next.
-//  * grouped_gemm_kernel (experts of up to 192 rows, 128 with fp8 weights, and with fp8 weights what an
-//    expert's full 256-row tiles leave over; work that mostly streams weights): one
+//  * grouped_gemm_kernel (experts of up to 192 rows, and with fp8 weights what an expert's full 256-row tiles
+//    leave over if that is at most 192 rows; work that mostly streams weights): one
 //    workgroup per tile, grid = upper bound on the tile count, surplus workgroups exit at once;
 //    the tile height (16 ... 192 rows in steps of 16) follows the expert, groups of 4 tiles go round-robin
-//    to the XCDs.  Its tiles run through the weight streamers (stream16_tile, stream8x_tile, stream8_tile):
+//    to the XCDs.  Its tiles run through the weight streamers (stream16_tile, stream8x_tile, stream8w_tile, stream8_tile):
 //    weights AND token rows reach LDS by DMA, three weight buffers, one barrier per stage.
 //
 // Workgroup = 8 waves, two per SIMD.  v_mfma_f32_16x16x32_bf16 throughout: on real (non-zero) data this
@@ -1034,13 +1034,186 @@ __device__ __forceinline__ void stream8x_tile(const GemmArgs& g, SBuf b0, SBuf b
     }
 }
 
-// M tiles of an expert with `count` rows in the one-workgroup-per-tile kernel: one tile of 64, 128 or (bf16 weights)
-// 192 rows if that holds them all, else tiles of 128.  The height follows the EXPERT, not the launch: a tile taller
+// ---- fp8 weight streamer in the persistent kernel's summation order: tiles of 129 to 192 rows ----
+//
+// stream8x_tile for 9 to 12 groups of 16 token rows: what an fp8 expert's full 256-row tiles leave over when that is
+// more than 128 rows (as a padded 256-row tile of the persistent kernel such rows cost a third to a half more matrix
+// work than they hold), and experts of that size in calls that this kernel serves alone.  Same weight DMA and LDS
+// layouts, the same division of labour (a weight is converted once, by the wave that multiplies it: with two sets of
+// 4 waves over the token groups, as in the bf16 streamer, every weight is converted twice, and the conversion then
+// takes the vector ALU as long as the products take the matrix cores -- DeepSeek-V3 at 4096 tokens 4.52 against 4.31
+// ms), same k values in the same lanes.  What differs: such a tile is bound by the matrix cores, not by the weight
+// stream, and 192 token rows x 64 k are 24 KiB, so there are two weight buffers, the next block requested right
+// after a block's first barrier (a block of 128 k takes the matrix cores about 2 us, more than a trip to memory), and
+// two token buffers, one per half of a block, each refilled right after the barrier that retires it, one half ahead
+// (token rows come out of L2).
+// Before a block's first half everything this wave requested must have landed (vmcnt 0); before its second half all
+// but the 4 weight instructions of the next block, which were issued behind that half's token rows.
+template <int TG, bool SWIGLU>   // TG: 16-row token groups multiplied (9 .. 12)
+__device__ __forceinline__ void stream8w_tile(const GemmArgs& g, uint8_t* w0, uint8_t* w1, uint8_t* t0, uint8_t* t1, int e,
+                                              int row0, int row_end, int n_tile, bool rotate) {
+    constexpr int NBLK = SWIGLU ? 128 : 256;
+    constexpr int NF = 2;                         // 16-row weight fragments per wave
+    constexpr int NDT = (2 * TG + 7) / 8;         // token DMA instructions per wave and half (8 rows each)
+    static_assert(TG >= 9 && TG <= 12 && NDT == 3, "token rows staged");
+    const int tid = threadIdx.x, lane = tid & 63, wave = uni(tid >> 6);
+    const int n0 = n_tile * NBLK;
+    const int K = g.K, N = g.N;
+    const int npair = K >> 7;
+    const int prot = rotate ? n_tile % npair : 0;             // k_rotation in blocks of 128 k
+
+    // ---- DMA coordinates (weights as in stream8x_tile: wave w brings LDS rows 32 w .. 32 w + 31, fragments 2 w, 2 w + 1) ----
+    const int lr = lane >> 3, pp = lane & 7;
+    uint32_t w_voff[4], t_voff[NDT];
+    const uint8_t* bmat[2];
+    cptr_f32 sc[2];
+    int srow[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        bmat[j] = uni_ptr((SWIGLU && j == 1) ? g.b1[e] : g.b0[e]);
+        sc[j] = (cptr_f32)(uintptr_t)uni_ptr((SWIGLU && j == 1) ? g.s1[e] : g.s0[e]);
+        srow[j] = min((n0 + (SWIGLU ? 0 : 32 * wave)) >> 7, (N >> 7) - 1) * npair;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int fr = 8 * (i & 1) + lr;
+        const int rt = SWIGLU ? 16 * wave + fr : 32 * wave + 16 * (i >> 1) + fr;      // row of the tile's N range
+        w_voff[i] = (uint32_t)min(n0 + rt, N - 1) * (uint32_t)K + (uint32_t)((pp ^ wsw(fr)) << 4);
+    }
+    const uint8_t* a_base = reinterpret_cast<const uint8_t*>(g.a) + (g.row_map ? (size_t)0 : (size_t)row0 * K * 2);
+    const int a_records = g.row_map ? (int)(uint32_t)g.a_bytes : (row_end - row0) * K * 2;
+#pragma unroll
+    for (int i = 0; i < NDT; ++i) {               // token rows 64 i + 8 wave + lr; rows past the tile's last: zeros, no request
+        const int tr = 64 * i + 8 * wave + lr;
+        const int r = min(row0 + tr, row_end - 1);
+        const int src = g.row_map ? ((gptr_i32)(uintptr_t)g.row_map)[r] : r - row0;
+        t_voff[i] = (uint32_t)src * (uint32_t)(K * 2) + (uint32_t)((pp ^ swz(tr)) << 4);
+        if (row0 + tr >= row_end || (g.row_map && (unsigned)src >= (unsigned)g.a_rows)) t_voff[i] = 0xfffffff0u;
+    }
+    float rsc[2][2];                              // block scales of the block being multiplied / of the next one
+    auto block_of = [&](int p_pipe) { int pr = min(p_pipe, npair - 1) + prot; return pr >= npair ? pr - npair : pr; };
+    auto scales = [&](int p_pipe, int set) {      // scalar loads (uniform addresses in the constant address space)
+        const int pr = block_of(p_pipe);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) rsc[set][j] = sc[j][srow[j] + pr];
+    };
+    auto dma_w = [&](int p_pipe, uint8_t* wb, int i) __attribute__((always_inline)) {
+        const int live = uni(p_pipe < npair ? -1 : 0);   // past the end: an empty descriptor, zeros without a request
+        const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)bmat[i >> 1], 0, live, 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_u8)(wb + wave * 4096 + i * 1024), 16, w_voff[i], (uint32_t)(block_of(p_pipe) * 128), 0, 2);
+    };
+    auto dma_t = [&](int hb_pipe, uint8_t* tb, int i) __attribute__((always_inline)) {
+        const int live = uni(hb_pipe < 2 * npair ? -1 : 0);
+        const int hb = min(hb_pipe, 2 * npair - 1);
+        const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)a_base, 0, live & a_records, 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_u8)(tb + (64 * i + 8 * wave) * 128), 16, t_voff[i],
+                                                 (uint32_t)(block_of(hb >> 1) * 256 + (hb & 1) * 128), 0, 0);
+    };
+
+    // ---- operand coordinates: a wave multiplies the two fragments it brought ----
+    const int frow = lane & 15, q = lane >> 4;
+    const int fq = ((q & 1) << 1) | (q >> 1);
+    const uint32_t wkey = (uint32_t)wsw(frow), tkey = (uint32_t)swz(frow);
+    const uint32_t w_rd = (uint32_t)(wave * 4096 + frow * 128), t_rd = (uint32_t)(frow * 128);
+    f32x4 acc[TG][NF];
+#pragma unroll
+    for (int t = 0; t < TG; ++t)
+#pragma unroll
+        for (int f = 0; f < NF; ++f) acc[t][f] = f32x4{0};
+
+    // Half h of block p: weights out of wb (block p), token rows out of tb (half 2 p + h).
+    auto half = [&](int p, int h, const uint8_t* wb, const uint8_t* tb, uint8_t* w_refill, uint8_t* t_refill, int sset) __attribute__((always_inline)) {
+        if (h == 0) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        // every wave has left half 2 p + h - 1 (its token buffer takes half 2 p + h + 1) and, h == 0, block p - 1 (its
+        // weight buffer takes block p + 1)
+#pragma unroll
+        for (int i = 0; i < NDT; ++i) dma_t(2 * p + h + 1, t_refill, i);
+        if (h == 0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dma_w(p + 1, w_refill, i);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        u32x2 wraw[2][NF];
+        bf16x8 tf[2][TG];
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+#pragma unroll
+            for (int f = 0; f < NF; ++f) {
+                // (the whole 16-byte part, of which this lane group uses one half and the group two further on the other)
+                const u32x4 part = *reinterpret_cast<const u32x4*>(wb + w_rd + f * 2048 + (((4 * h + 2 * s2 + (fq >> 1)) ^ wkey) << 4));
+                wraw[s2][f] = (fq & 1) ? u32x2{part[2], part[3]} : u32x2{part[0], part[1]};
+            }
+            const uint32_t coff = (uint32_t)(((4 * s2 + fq) ^ tkey) << 4);
+#pragma unroll
+            for (int t = 0; t < TG; ++t) tf[s2][t] = *reinterpret_cast<const bf16x8*>(tb + t_rd + t * 16 * 128 + coff);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            bf16x8 wa[NF];
+#pragma unroll
+            for (int f = 0; f < NF; ++f)
+                wa[f] = __builtin_bit_cast(bf16x8, dequant8(wraw[s2][f][0], wraw[s2][f][1], rsc[sset][f]));
+#pragma unroll
+            for (int t = 0; t < TG; ++t)
+#pragma unroll
+                for (int f = 0; f < NF; ++f) acc[t][f] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[f], tf[s2][t], acc[t][f], 0, 0, 0);
+        }
+        // (the next block's scales: scalar loads, issued where no LDS read is outstanding)
+        if (h == 0) scales(p + 1, sset ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    scales(0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_w(0, w0, i);
+#pragma unroll
+    for (int i = 0; i < NDT; ++i) dma_t(0, t0, i);
+    // Two blocks bring the weight buffers and the scale sets back to where they started: literal buffers in the loop body.
+    int p = 0;
+    for (; p + 2 <= npair; p += 2) {
+        half(p, 0, w0, t0, w1, t1, 0);
+        half(p, 1, w0, t1, w1, t0, 0);
+        half(p + 1, 0, w1, t0, w0, t1, 1);
+        half(p + 1, 1, w1, t1, w0, t0, 1);
+    }
+    if (p < npair) {
+        half(p, 0, w0, t0, w1, t1, 0);
+        half(p, 1, w0, t1, w1, t0, 0);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no DMA may land in LDS after the workgroup has gone
+
+    // ---- epilogue: a lane holds 4 consecutive columns of one row per accumulator and stores them itself ----
+#pragma unroll
+    for (int t = 0; t < TG; ++t) {
+        const int r = row0 + 16 * t + frow;
+        if (r >= row_end) continue;
+#pragma unroll
+        for (int f = 0; f < (SWIGLU ? 1 : NF); ++f) {
+            const int col = n0 + (SWIGLU ? 16 : 32) * wave + 16 * f + 4 * q;
+            if (col < N) *reinterpret_cast<u32x2*>(g.c + (size_t)r * N + col) = epilogue_pack<SWIGLU>(acc[t][f], acc[t][SWIGLU ? 1 : f]);
+        }
+    }
+}
+
+template <bool SWIGLU>
+__device__ __forceinline__ void stream8w(const GemmArgs& g, uint8_t* w0, uint8_t* w1, uint8_t* t0, uint8_t* t1, int e, int row0,
+                                         int row_end, int n_tile, bool rotate) {
+    const int rows = row_end - row0;
+    if (rows <= 144) stream8w_tile<9, SWIGLU>(g, w0, w1, t0, t1, e, row0, row_end, n_tile, rotate);
+    else if (rows <= 160) stream8w_tile<10, SWIGLU>(g, w0, w1, t0, t1, e, row0, row_end, n_tile, rotate);
+    else if (rows <= 176) stream8w_tile<11, SWIGLU>(g, w0, w1, t0, t1, e, row0, row_end, n_tile, rotate);
+    else stream8w_tile<12, SWIGLU>(g, w0, w1, t0, t1, e, row0, row_end, n_tile, rotate);
+}
+
+// M tiles of an expert with `count` rows in the one-workgroup-per-tile kernel: one tile of up to 192 rows if that
+// holds them all, else tiles of 128.  The height follows the EXPERT, not the launch: a tile taller
 // than its expert stages and multiplies rows that do not exist, and an expert cut into several tiles reads its
 // weights once per tile and adds workgroups (the hot expert of a skewed decode batch: 9 x 128 tiles are 4.5 rounds
-// of 256 CUs and cost 5).  The tiles of an expert that is cut (above 192 rows; above 128 with fp8 weights, where the
-// 192-row body does not fit the registers) run side by side on one XCD and take the weights with plain loads, so
-// that all but the first read of a line come out of that XCD's L2.
+// of 256 CUs and cost 5).  The tiles of an expert that is cut (above 192 rows) run side by side on one XCD and take
+// the weights with plain loads, so that all but the first read of a line come out of that XCD's L2.
 // 256-row tiles of an expert with `count` rows in the persistent kernel's tile space
 // whether an expert of `count` rows belongs to the one-workgroup-per-tile kernel (no rem_split)
 __device__ __forceinline__ bool is_cold(const GemmArgs& g, int count) {
@@ -1067,8 +1240,9 @@ __device__ __forceinline__ int tail_tiles(const GemmArgs& g, int total, int own)
     return move < keep ? tail : 0;
 }
 
-template <int SINGLE>   // rows that one tile may hold
+template <bool PAIR>   // whether an expert of PAIR_LO .. PAIR_HI rows is cut in the middle (bf16 weights)
 __device__ __forceinline__ int tiles_of(int count) {
+    constexpr int SINGLE = 192;   // rows that one tile may hold
     if (count <= SINGLE) return count > 0 ? 1 : 0;
     // bf16 weights: an expert of 257 to 384 rows is cut in the middle, into two tiles of the 192-row body that run
     // side by side on one XCD and share the weights through its L2: 320 rows are 2 x 160 rows of MFMA work, where
@@ -1076,7 +1250,7 @@ __device__ __forceinline__ int tiles_of(int count) {
     // Mixtral-8x22B shapes, 8 experts of 288 / 320 / 384 rows: gate/up 1.31 / 1.29 / 1.30 -> 1.07 / 1.13 / 1.17 ms,
     // down projection within 4 % either way; up to 256 rows one tile of the persistent kernel stays better (224
     // rows: 0.82 against 1.01 ms).
-    if (SINGLE == 192 && count > PAIR_LO - 1 && count <= PAIR_HI) return 2;
+    if (PAIR && count > PAIR_LO - 1 && count <= PAIR_HI) return 2;
     return (count + 127) >> 7;
 }
 // rows of either tile of such a pair (the first tile holds whole 16-row groups)
@@ -1086,7 +1260,7 @@ __device__ __forceinline__ int half_rows(int count) { return ((count + 1) / 2 + 
 template <bool W8>
 __device__ __forceinline__ int own_tiles(const GemmArgs& g, int c) {
     if (g.rem_split) c &= 255;      // the rows the persistent kernel's full tiles leave over
-    return (g.rem_split ? c > g.cold_max : !is_cold(g, c)) ? 0 : tiles_of<(W8 ? 128 : 192)>(c);
+    return (g.rem_split ? c > g.cold_max : !is_cold(g, c)) ? 0 : tiles_of<!W8>(c);
 }
 
 // sum over the experts of f(count) (every thread gets it; two barriers)
@@ -1289,16 +1463,17 @@ __device__ __forceinline__ void stream8x(const GemmArgs& g, SBuf b0, SBuf b1, SB
 template <int WN, bool SWIGLU, bool W8>
 __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     constexpr int NT = 128 * WN;
-    // Three weight arrays of 32 KiB and token arrays of 16 KiB (fp8 weights: three, 128 rows) or 24 KiB (bf16: two,
-    // 192 rows) -- the buffers of the weight streamers, written by DMA, as separate objects so that a read of one
-    // waits for no DMA into another; gemm_tile's two stages (up to 128 token rows + 256 weight rows) are two pairs
-    // of them.
+    // Three weight arrays of 32 KiB and token arrays of 16 KiB (fp8 weights: three, 128 rows; the second one 24 KiB)
+    // or 24 KiB (bf16: two, 192 rows) -- the buffers of the weight streamers, written by DMA, as separate objects so
+    // that a read of one waits for no DMA into another; gemm_tile's two stages (up to 128 token rows + 256 weight
+    // rows) are two pairs of them.  The fp8 streamer for 129 to 192 rows has two weight buffers and keeps its token
+    // rows (24 KiB per half) in the third weight array and the 24 KiB token array.
     constexpr int TB = W8 ? 128 * ROW_B : 192 * ROW_B;
     __shared__ __attribute__((aligned(1024))) uint8_t lw0[S8_WBYTES];
     __shared__ __attribute__((aligned(1024))) uint8_t lw1[S8_WBYTES];
     __shared__ __attribute__((aligned(1024))) uint8_t lw2[S8_WBYTES];
     __shared__ __attribute__((aligned(1024))) uint8_t lt0[TB];
-    __shared__ __attribute__((aligned(1024))) uint8_t lt1[TB];
+    __shared__ __attribute__((aligned(1024))) uint8_t lt1[192 * ROW_B];
     __shared__ __attribute__((aligned(1024))) uint8_t lt2[W8 ? TB : 16];
     static_assert(S8_TROWS * 256 <= 128 * ROW_B && S8_WBYTES == BN_ROWS * ROW_B, "regions of a streamer buffer");
     auto stage = [&](int i) { return Stage{i ? lt1 : lt0, i ? lw1 : lw0, i ? lw1 : lw0}; };
@@ -1377,7 +1552,7 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
     if (W8 && s8_ok) {
         // fp8 weights: the weight streamers.  Up to 64 rows in a call that this kernel has to itself, where no other
         // kernel's summation order has to be matched: the form that reads a lane's 16 weights at once.  Everything
-        // else -- up to 128 rows; what an expert's full 256-row tiles leave over; 128-row slices of larger experts
+        // else -- up to 192 rows; what an expert's full 256-row tiles leave over; 128-row slices of larger experts
         // when the kernel is alone -- in the persistent kernel's order.
         const int r0 = first_row + (mt_e > 1 ? m_tile * 128 : 0), r1 = mt_e > 1 ? min(row_end, r0 + 128) : row_end;
         const int rows = r1 - r0;
@@ -1386,12 +1561,14 @@ __global__ __launch_bounds__(128 * WN) void grouped_gemm_kernel(GemmArgs g) {
             else if (rows <= 32) stream8_tile<2, SWIGLU>(g, sb0, sb1, sb2, e, r0, r1, n_tile);
             else if (rows <= 48) stream8_tile<3, SWIGLU>(g, sb0, sb1, sb2, e, r0, r1, n_tile);
             else stream8_tile<4, SWIGLU>(g, sb0, sb1, sb2, e, r0, r1, n_tile);
+        } else if (rows > 128) {                 // (one tile of 129 to 192 rows)
+            stream8w<SWIGLU>(g, lw0, lw1, lw2, lt1, e, r0, r1, n_tile, alone);
         } else {
             stream8x<SWIGLU>(g, sb0, sb1, sb2, e, r0, r1, n_tile, alone);
         }
         return;
     }
-    // The rows of this workgroup: the expert's (one tile: up to 192 rows, 128 with fp8 weights), one half of an
+    // The rows of this workgroup: the expert's (one tile: up to 192 rows), one half of an
     // expert of PAIR_LO .. PAIR_HI rows (bf16), or a 128-row slice.
     const int rows_e = row_end - first_row;
     const bool pair = !W8 && rows_e >= PAIR_LO && rows_e <= PAIR_HI;
@@ -1817,11 +1994,14 @@ int launch_mt(const GemmArgs& g0, int n_rows, hipStream_t st) {
     // last tile costs the persistent kernel a full tile of MFMA time; the other kernel streams the expert's weights
     // once more for it, and fp8 weights are half the bytes.  DeepSeek-V3, 65536 tokens (256 experts of 581 ... 3941
     // rows, every second one with at most 128 rows over): block step 46.3 -> 45.8 ms, routed gate/up 25.2 -> 24.8,
-    // down 12.9 -> 12.7 (with up to 64 or 96 rows over 46.2 - 46.3; with all, as two 128-row tiles, 47.1).  With bf16
+    // down 12.9 -> 12.7 (with up to 64 or 96 rows over 46.2 - 46.3; with all, as two 128-row tiles, 47.1).  Up to 192
+    // rows over, on the streamer form for 129 to 192 rows: the headline step stays (45.95 -> 45.85), DeepSeek-V3 at
+    // 3584 / 4096 / 8192 tokens 4.53 -> 3.99, 4.64 -> 4.31, 7.50 -> 7.41 ms (at 4096 tokens 109 of the 256 experts hold
+    // 129 to 192 rows, which were padded 256-row tiles).  With bf16
     // weights it is break-even (Mixtral-8x7B 9.28 -> 9.23 ms, DeepSeek-V2-236B 11.34 -> 11.42) and not done.
     // (Both launches at every mean: from 1536 rows per expert a small expert is rare, but the second launch is there
     // for the persistent kernel's last round anyway.)
-    g.cold_max = W8 ? 128 : 192;
+    g.cold_max = 192;
     g.rem_split = W8 ? 1 : 0;
     g.pair_rows = W8 ? 0 : 1;
     // Last round of the persistent kernel (tail_tiles above): Mixtral-8x22B, 8192 tokens, down projection (6.4 rounds

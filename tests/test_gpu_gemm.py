@@ -331,6 +331,49 @@ def test_bf16_weight_streamer_shapes_and_gather(h, I):
     assert rel_max(y, ref32) <= TOL and rel_max(y, refr) <= TOL
 
 
+@pytest.mark.parametrize("counts", [
+    [129, 144, 145, 160, 176, 177, 192, 400, 600, 320, 449, 70],     # mean 255: both kernels; 400 = 256 + 144 left over
+    [129, 150, 192, 170, 64, 65] + [5] * 20])                         # mean 35: the one-workgroup-per-tile kernel alone
+@pytest.mark.parametrize("h,I", [(640, 384), (1024, 896)])            # 5 / 3 and 8 / 7 blocks of 128 k (odd and even counts)
+def test_fp8_weight_streamer_tiles_of_129_to_192_rows(counts, h, I):
+    """fp8 tiles of 129 to 192 rows -- experts of that size, and what the full 256-row tiles of a larger one leave over
+    -- run on the streamer form with two weight buffers and 24 KiB of token rows per half.  Experts that share one set
+    of weights and start with the same five rows: those rows come out bit-identical from every tile height, in the
+    first list also from the persistent kernel (600 = 2 x 256 + 88 rows, 449 = 256 + 193) and the 128-row form (320 =
+    256 + 64); the call gives the same bits every time, and the rows are within the layer bound of the oracle."""
+    from moe_gen_amd import ops
+    E = len(counts)
+    print(f"fp8 streamer 129-192 h={h} I={I} counts={counts}", flush=True)
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    n = int(offsets[-1])
+    g = torch.Generator().manual_seed(297)
+    x = torch.randn(n, h, generator=g).to(torch.bfloat16)
+    for e in range(1, E):
+        x[offsets[e]:offsets[e] + 5] = x[:5]
+    one = make_experts(1, h, I, True, 298)[0]
+    dm = [tuple(t.cuda() for t in m) for m in one]
+    ptrs = ops.expert_pointers([dm[0][0]] * E, [dm[1][0]] * E, [dm[2][0]] * E, [dm[0][1]] * E, [dm[1][1]] * E, [dm[2][1]] * E)
+    off_d = torch.from_numpy(offsets).cuda()
+    xd = x.cuda()
+    ys = [ops.grouped_swiglu(xd, None, ptrs, off_d, n).clone() for _ in range(6)]
+    rm = torch.randperm(n, generator=g).to(torch.int32)
+    xin = torch.empty_like(x)
+    xin[rm.long()] = x
+    y_map = ops.grouped_swiglu(xin.cuda(), rm.cuda(), ptrs, off_d, n)       # the same rows gathered through a row map
+    torch.cuda.synchronize()
+    for rep in range(1, 6):
+        assert torch.equal(ys[rep], ys[0]), f"call {rep} differs from call 0"
+    assert torch.equal(y_map, ys[0])
+    alone = n // E < 128
+    for e in range(1, E):
+        if alone and counts[e] <= 64:
+            continue        # (alone, up to 64 rows: the streamer form with its own order of summation)
+        assert torch.equal(ys[0][offsets[e]:offsets[e] + 5], ys[0][:5]), f"expert {e} ({counts[e]} rows)"
+    wg, wu, wd = (f32_of(m) for m in one)
+    ref = O.mlp_f32(O.bf16_to_f32(bits(x)), wg, wu, wd)
+    assert rel_max(O.bf16_to_f32(bits(ys[0])), ref) <= TOL
+
+
 @pytest.mark.parametrize("h,I", [(512, 640), (640, 896), (896, 512)])      # 4 / 5 / 7 blocks of 128 k (gate/up), 5 / 7 / 4 (down)
 def test_fp8_weight_streamer_shapes_and_gather(h, I):
     """The fp8 weight streamer on every token-group count and both sides of each boundary, with block counts that
