@@ -354,7 +354,7 @@ def calibrate(w, reps: int = 40):
 # (two runs; FETCH_SIZE scaled by 2.0, the factor a plain copy kernel of known size showed on this
 # box, WRITE_SIZE by 1.0).  bench.py cannot run the profiler on itself: these are RECORDED figures,
 # copied from the named summary under profiles/, for the workloads that were profiled; None elsewhere.
-MEASURED_TRAFFIC = {"deepseek_v3_w8a16": (22.5e9, "profiles/pmc_traffic_deepseek_v3_w8a16_65536.md"),
+MEASURED_TRAFFIC = {"deepseek_v3_w8a16": (23.7e9, "profiles/pmc_traffic_deepseek_v3_w8a16_65536.md"),
                     # 3.03 GiB fetched + the 16 MiB of activations written
                     "mixtral_8x22b_decode": (3.27e9, "profiles/pmc_small_workloads_decode_and_v2_lite.md")}
 
