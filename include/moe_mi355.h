@@ -160,10 +160,10 @@ int moe_dispatch_static(const int32_t* topk_idx, int32_t n_tokens, int32_t top_k
  *   phases    MOE_PHASE_GATE_UP (writes act), MOE_PHASE_DOWN (reads act, writes y) or
  *             MOE_PHASE_BOTH; the two launches can be issued (and timed) separately
  * Requires h % 64 == 0 and I % 64 == 0, 1 <= E <= 1024.  Two kernels share a call: experts that fit one tile of
- * up to 128 or (bf16 weights) 192 rows run one workgroup per tile, at a tile height chosen per expert on the device
- * in steps of 16 rows (bf16: also experts of 257 to 384 rows, as two such tiles);
+ * up to 192 rows run one workgroup per tile, at a tile height chosen per expert on the device in steps of 16 rows
+ * (bf16 weights: also experts of 257 to 384 rows, as two such tiles);
  * larger experts run on 256-row tiles of persistent workgroups (with fp8 weights: their full 256-row tiles, and the
- * rows these leave over as one small tile of the first kind if they are at most 128).  The persistent workgroups,
+ * rows these leave over as one tile of the first kind if they are at most 192).  The persistent workgroups,
  * one per CU, take whole rounds of tiles; a last, partial round is cut into 128-row halves and runs with the first
  * kind when that shortens the two launches (alone: if it is at most half the CUs' worth of tiles).  Below a mean of 128 rows per expert (n_rows / E), with K not a multiple of
  * 128, with more than 512 experts or with 4 GiB or more of gathered x, the one-workgroup-per-tile kernel serves the
