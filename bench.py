@@ -379,7 +379,7 @@ def run_workload(name: str, args, with_cpu: bool):
     mean_rows = w.n * w.k // w.E
     # which kernels a grouped GEMM call launches follows from the mean rows per expert (grouped_gemm.hip, launch_mt):
     # below 128 the one-workgroup-per-tile kernel alone; else both (on the former, bf16: experts of up to 192 rows;
-    # fp8: what an expert's full 256-row tiles leave over, if at most 128 rows; either: the persistent kernel's last
+    # fp8: what an expert's full 256-row tiles leave over, if at most 192 rows; either: the persistent kernel's last
     # round of tiles if it is at most half a round; most rows, and the time, on the latter)
     persistent = mean_rows >= 128 and w.E <= 512 and w.h % 128 == 0
     # yardsticks of this box, taken right before and right after the timed passes (MFMA-bound workloads)

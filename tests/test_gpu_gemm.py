@@ -113,7 +113,7 @@ def test_grouped_odd_stage_counts(E, h, I, counts):
 def test_tile_height_follows_the_expert(fp8):
     """One launch of the one-workgroup-per-tile kernel alone (mean rows per expert below 128) with experts on both
     sides of every tile-height boundary: a 64-row tile up to 64 rows, one 128-row tile up to 128, one 192-row
-    tile up to 192 (bf16 weights only), several 128-row tiles above (those read their weights with plain loads).
+    tile up to 192, several 128-row tiles above (those share their weights through one XCD's L2).
     Against the oracle, and an expert's rows bit-for-bit against a launch that holds this expert alone."""
     from moe_gen_amd import ops
     E, h, I = 16, 512, 384
@@ -144,8 +144,8 @@ def test_experts_split_between_the_two_kernels(fp8):
     """From a mean of 128 rows per expert a call launches both kernels and every expert goes by its own count.  bf16
     weights: up to 192 rows one tile of the one-workgroup-per-tile kernel, more the persistent kernel's 256-row tiles.
     fp8 weights: the persistent kernel's tile space holds an expert's full 256-row tiles, and what they leave over goes
-    to the other kernel if it is at most 128 rows (300 = 256 + 44, 640 = 512 + 128, 512 leaves nothing, 700 = 512 + 188
-    stays whole).  (At this size the tile space is a short last round, which the other kernel runs as half tiles.)
+    to the other kernel if it is at most 192 rows (300 = 256 + 44, 640 = 512 + 128, 700 = 512 + 188, 512 leaves nothing,
+    2000 = 1792 + 208 stays whole).  (At this size the tile space is a short last round, which the other kernel runs as half tiles.)
     Against the oracle, and every expert's rows bit-for-bit against a call that holds this expert alone, whichever
     kernel and tile its rows fall to there.  (A lone call below a mean of 128 is served by the one-workgroup-per-tile
     kernel alone, which then walks k from other stages than a call of both kernels, and is left out.)"""
@@ -604,6 +604,34 @@ def test_persistent_kernel_corner_shapes(fp8, E, h, I, counts):
     print(f"persistent corners fp8={fp8} E={E} h={h} I={I}", flush=True)
     y, ref32, _ = run_case(E, h, I, counts, fp8, seed=37, use_row_map=True)
     assert np.isfinite(y).all() and rel_max(y, ref32) <= TOL
+
+
+EDGE_COUNTS = [0, 1, 17, 64, 65, 128, 129, 144, 145, 160, 161, 192, 193, 256, 257, 300, 384, 385, 449, 700]
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("seed", range(10))
+def test_grouped_seeded_mixtures(fp8, seed):
+    """Seeded draws of expert count, sizes and per-expert rows from both sides of every tile-height and
+    kernel boundary (64 / 128 / 144 / 160 / 192 / 256 / 384 rows), with and without a row map: whichever
+    kernels and tile forms the launcher picks for the mixture, every row matches the oracle, and a second
+    call returns the same bits."""
+    rng = np.random.default_rng(1000 + seed)
+    E = int(rng.choice([1, 2, 3, 5, 8, 13]))
+    h, I = 128 * int(rng.integers(1, 6)), 128 * int(rng.integers(1, 6))
+    kind = ["few", "middle", "edges", "many"][seed % 4]
+    counts = {"few": rng.integers(0, 70, E), "middle": rng.integers(100, 400, E),
+              "edges": rng.choice(EDGE_COUNTS, E), "many": rng.integers(300, 900, E)}[kind]
+    counts = [int(c) for c in counts]
+    if sum(counts) == 0:
+        counts[0] = 33
+    use_map = bool(rng.integers(0, 2))
+    print(f"mixture fp8={fp8} seed={seed} E={E} h={h} I={I} {kind} row_map={use_map} counts={counts}", flush=True)
+    y, ref32, refr = run_case(E, h, I, counts, fp8, seed=300 + seed, use_row_map=use_map)
+    y2, _, _ = run_case(E, h, I, counts, fp8, seed=300 + seed, use_row_map=use_map)
+    assert np.isfinite(y).all()
+    assert rel_max(y, ref32) <= TOL and rel_max(y, refr) <= TOL
+    assert np.array_equal(y, y2)
 
 
 @pytest.mark.parametrize("n_src,n", [(300, 600), (60, 120)])
