@@ -312,7 +312,6 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, Stage st0, Stage st
                                           int n_tile) {
     constexpr int NT = 128 * WN;                // threads
     constexpr int BM = 64 * MT;                 // rows per workgroup
-    constexpr int A_STAGE = BM * ROW_B;         // bytes
     constexpr int RA = NT / 8;                  // A rows covered by one pass of the workgroup
     constexpr int NA = BM / RA;                 // 16-byte A chunks per thread per stage
     constexpr int RB = NT / 8;                  // B rows per pass of the workgroup (8 lanes per 128-byte row)
@@ -664,7 +663,6 @@ __device__ __forceinline__ int tsw(int r) { return (r & 3) | ((r & 4) << 1); }
 
 constexpr int S8_WBYTES = 32 * 1024;              // weight region of a buffer: 8 waves x 32 rows x 128 fp8
 constexpr int S8_TROWS = 64;                      // token rows staged
-constexpr int S8_BUF = S8_WBYTES + S8_TROWS * 256;
 
 // A buffer of the weight streamers: the weight region and the token region are separate LDS arrays, so that a read of
 // one never has to wait for a DMA into the other
