@@ -644,6 +644,194 @@ __global__ __launch_bounds__(64) void router_pair_kernel(
     }
 }
 
+// Fourth logit engine, for more than 64 experts and few tokens (a decode or small prefill batch of DeepSeek-V2 /
+// V3): the 4 x 64 layout of the 4x4 MFMA (4 tokens per workgroup, a wave per 64 experts, lane l of a wave the
+// expert 64 wave + l) without a workgroup-wide stage.  Under router_kernel every workgroup of 4 tokens converts the
+// whole gate matrix to fp32 and passes it through LDS between two barriers per 64 k: 64 KiB of LDS stores and 128 KiB
+// of reads per stage, more LDS time than the 64 MFMAs of the stage take.  Here a wave works alone:
+//  * the 128-byte lines of ITS 64 gate rows reach its own LDS region as bf16 by DMA (8 instructions per 64 k; chunk c
+//    of row r in 16-byte slot c ^ g(r), so that the 16 lanes the LDS serves together -- rows 8i .. 8i+7 and
+//    32+8i .. 39+8i -- fall on 16 different bank groups); a lane reads the 8 weights of its expert with one
+//    ds_read_b128 and widens them to fp32 between the MFMAs (a shift or a mask each);
+//  * the token values never touch LDS: the MFMA broadcasts the A operand of one block to all 16, so a register that
+//    holds the 4 tokens' values of 16 consecutive k (one 2-byte load per lane) feeds 16 instructions;
+//  * one wave's LDS reads execute in order and its DMA is ordered by vmcnt, so the k loop has no barrier.
+// Each logit is the same chain of one fused multiply-add per k as in every other engine.  Per k a wave issues one
+// MFMA, one conversion and an eighth of a 16-byte LDS read: 11.9 ns (DeepSeek-V3, up to 1024 tokens: 97 ... 106 us
+// for h = 7168, from 165 ... 178); 9.7 ns without the conversion and 8.3 ns without the LDS read either, which is
+// the MFMA chain itself.
+typedef __attribute__((address_space(3))) uint8_t* lds_u8;
+__device__ __forceinline__ int thin_slot(int r) { return ((r >> 1) & 3) | (((r >> 5) & 1) << 2); }
+
+// The A operand of block B is broadcast to all 16 blocks of the instruction (cbsz = 4, abid = B), so ONE register holds
+// the token values of 16 consecutive k: lanes 4b .. 4b+3 the 4 tokens at k0 + b.  The B operand of lane l is expert l
+// of the wave's 64.
+template <int B>
+__device__ __forceinline__ f32x4 mfma_4_tokens(float a, float b, f32x4 acc) {
+    return __builtin_amdgcn_mfma_f32_4x4x1f32(a, b, acc, 4, B, 0);
+}
+
+// NBUF: weight buffers per wave (3: two stages in flight, one workgroup per CU; 2: one stage in flight and at most
+// 256 registers, two workgroups per CU).
+template <int WE, int NBUF>
+__global__ __launch_bounds__(64 * WE, NBUF == 2 ? 2 : 1) void router_thin_kernel(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ wg, const float* __restrict__ bias,
+    moe_router_params p, int32_t* __restrict__ topk_idx, float* __restrict__ topk_w, float* __restrict__ logits_out) {
+    constexpr int KC = 64, BT = 4, EP = 64 * WE, WBYTES = 64 * 128;
+    // one array per weight buffer: a read of one then never waits for the DMA in flight into another
+    __shared__ __attribute__((aligned(1024))) uint8_t wb0[WE * WBYTES];           // written by DMA only
+    __shared__ __attribute__((aligned(1024))) uint8_t wb1[WE * WBYTES];
+    __shared__ __attribute__((aligned(1024))) uint8_t wb2[NBUF == 3 ? WE * WBYTES : 1024];
+    __shared__ __attribute__((aligned(16))) float lg[BT * EP];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n = p.n_tokens, h = p.hidden, E = p.n_experts;
+    const int t0 = blockIdx.x * BT;
+    const int nfull = h / KC, rem8 = (h % KC) / 8, nstage = nfull + (rem8 ? 1 : 0);
+
+    // weight DMA: instruction i brings rows 8i .. 8i+7 of the wave's 64, a lane the chunk that belongs in its slot
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void*)wg, 0, E * h * 2, 0x00020000);
+    int w_voff[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int r = 8 * i + (lane >> 3), c = (lane & 7) ^ thin_slot(r);
+        w_voff[i] = (min(64 * wave + r, E - 1) * h + c * 8) * 2;
+    }
+    auto dma_w = [&](uint8_t* buf, int st) {
+        uint8_t* dst = buf + wave * WBYTES;
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_u8)(dst + i * 1024), 16, w_voff[i], (uint32_t)(st * (KC * 2)), 0, 0);
+    };
+    // token values straight from memory into the broadcast layout: register g of a stage holds, in lanes
+    // 4b .. 4b+3, element 16 g + b of the 4 tokens (one 2-byte load per lane and 16 k), widened when its 16 k come up
+    const uint16_t* const xlane = x + (size_t)min(t0 + (lane & 3), n - 1) * h + (lane >> 2);
+    uint32_t xr[2][4];
+    auto load_x = [&](int set, int st) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int k = st * KC + 16 * g;
+            xr[set][g] = xlane[k + (lane >> 2) < h ? k : 0];
+        }
+    };
+
+    f32x4 acc = {0, 0, 0, 0};                  // register i: token i, expert 64 wave + lane
+    int w_roff[8];                             // chunk c of the lane's row inside a buffer
+#pragma unroll
+    for (int c = 0; c < 8; ++c) w_roff[c] = wave * WBYTES + lane * 128 + ((c ^ thin_slot(lane)) << 4);
+
+    auto wf = [](const u32x4& v, int j) {      // element j of 8 bf16 as fp32
+        return __uint_as_float((j & 1) ? (v[j >> 1] & 0xffff0000u) : (v[j >> 1] << 16));
+    };
+    // Stage st; the register set st & 1 and the buffers are literals at every call site.  The loads of stage
+    // st + NBUF - 1 (weights) and st + 2 (tokens) leave first, then the wait that lets the vector-memory operations
+    // younger than the DMA of stage st stay in flight (per stage ahead 8 DMA and 4 token loads).
+    auto stage = [&](int st, int set, const uint8_t* wb, uint8_t* wb_refill, int nch) {
+        uint32_t xs[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) xs[g] = xr[set][g];
+        load_x(set, min(st + 2, nstage - 1));
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the reads of stage st - 1, a stage old, before their buffer is refilled
+        dma_w(wb_refill, min(st + NBUF - 1, nstage - 1));
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NBUF - 1) * (8 + 4)) : "memory");
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            if (2 * g >= nch) break;
+            const u32x4 w0 = *reinterpret_cast<const u32x4*>(wb + w_roff[2 * g]);
+            const u32x4 w1 = *reinterpret_cast<const u32x4*>(wb + w_roff[2 * g + 1]);
+            const float xa = __uint_as_float(xs[g] << 16);
+#define MOE_THIN_K(B) \
+    if (2 * g + ((B) >> 3) < nch) acc = mfma_4_tokens<B>(xa, wf((B) < 8 ? w0 : w1, (B) & 7), acc);
+            MOE_THIN_K(0) MOE_THIN_K(1) MOE_THIN_K(2) MOE_THIN_K(3) MOE_THIN_K(4) MOE_THIN_K(5) MOE_THIN_K(6) MOE_THIN_K(7)
+            MOE_THIN_K(8) MOE_THIN_K(9) MOE_THIN_K(10) MOE_THIN_K(11) MOE_THIN_K(12) MOE_THIN_K(13) MOE_THIN_K(14) MOE_THIN_K(15)
+#undef MOE_THIN_K
+        }
+    };
+
+    int st = 0;
+    if constexpr (NBUF == 2) {
+        load_x(0, 0);
+        load_x(1, min(1, nstage - 1));
+        dma_w(wb0, 0);
+        for (; st + 2 <= nfull; st += 2) {
+            stage(st, 0, wb0, wb1, 8);
+            stage(st + 1, 1, wb1, wb0, 8);
+        }
+        const int left = nfull - st;
+        if (left > 0) stage(st, 0, wb0, wb1, 8);
+        if (rem8) {
+            if (left == 0) stage(st, 0, wb0, wb1, rem8);
+            else stage(st + 1, 1, wb1, wb0, rem8);
+        }
+    } else {
+        load_x(0, 0);
+        dma_w(wb0, 0);
+        load_x(1, min(1, nstage - 1));
+        dma_w(wb1, min(1, nstage - 1));
+        for (; st + 6 <= nfull; st += 6) {
+            stage(st, 0, wb0, wb2, 8);
+            stage(st + 1, 1, wb1, wb0, 8);
+            stage(st + 2, 0, wb2, wb1, 8);
+            stage(st + 3, 1, wb0, wb2, 8);
+            stage(st + 4, 0, wb1, wb0, 8);
+            stage(st + 5, 1, wb2, wb1, 8);
+        }
+        // up to 5 whole stages and one of fewer than 64 k are left; stage st + i has the literals of i
+        const int left = nfull - st;
+        if (left > 0) stage(st, 0, wb0, wb2, 8);
+        if (left > 1) stage(st + 1, 1, wb1, wb0, 8);
+        if (left > 2) stage(st + 2, 0, wb2, wb1, 8);
+        if (left > 3) stage(st + 3, 1, wb0, wb2, 8);
+        if (left > 4) stage(st + 4, 0, wb1, wb0, 8);
+        if (rem8) {
+            if (left == 0) stage(st, 0, wb0, wb2, rem8);
+            else if (left == 1) stage(st + 1, 1, wb1, wb0, rem8);
+            else if (left == 2) stage(st + 2, 0, wb2, wb1, rem8);
+            else if (left == 3) stage(st + 3, 1, wb0, wb2, rem8);
+            else if (left == 4) stage(st + 4, 0, wb1, wb0, rem8);
+            else stage(st + 5, 1, wb2, wb1, rem8);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // no DMA may land in LDS after the workgroup has gone
+
+#pragma unroll
+    for (int i = 0; i < 4; ++i) lg[i * EP + 64 * wave + lane] = acc[i];
+    __syncthreads();
+    for (int tb = wave; tb < BT; tb += WE) {
+        if (t0 + tb >= n) break;
+        const int t = t0 + tb;
+        route_token<64, WE>(lg + tb * EP, bias, p, topk_idx + (size_t)t * p.top_k, topk_w + (size_t)t * p.top_k,
+                            logits_out ? logits_out + (size_t)t * E : nullptr, true);
+    }
+}
+
+template <int WE, int NBUF>
+int launch_thin_as(const void* x, const void* w, const float* bias, const moe_router_params& p, int32_t* idx, float* tw,
+                   float* lo, hipStream_t st) {
+    hipLaunchKernelGGL((router_thin_kernel<WE, NBUF>), dim3((p.n_tokens + 3) / 4), dim3(64 * WE), 0, st,
+                       (const uint16_t*)x, (const uint16_t*)w, bias, p, idx, tw, lo);
+    MOE_HIP_CHECK(hipGetLastError());
+    return MOE_OK;
+}
+// Which calls the engine above serves.  On this chip a 4x4x1 MFMA keeps its wave for about 16 cycles whether or not
+// the next one depends on it, and two waves of a SIMD share the matrix core (two chains in one wave took 1.75 times
+// as long as one, two workgroups per CU 1.5 times), so once every CU has two workgroups the engines with more tokens
+// per instruction win.  Up to 1024 tokens: one workgroup per CU, three buffers.  Up to 2048 tokens and above 128
+// experts: two workgroups per CU, two buffers.  Measured (us, router_kernel -> this; h = 7168 / 5120):
+//   256 experts:  64 ... 1024 tokens 165 ... 178 -> 97 ... 106;  2048 tokens 232 -> 171;  3072: 235 against 258
+//   160 experts:  1024 tokens 96 -> 78;  2048 tokens 134 -> 118;  3072: 138 against 153
+//   128 experts:  1024 tokens 91 -> 77;  2048: 98 against 114
+// (a 16-token form on v_mfma_f32_16x16x1_4b_f32, 32 cycles per k by the book, ran at 77: 304 us at 4096 tokens of
+// 256 experts against 248; with two workgroups per CU 410 against 474 at 8192 tokens and behind again from 12288: not kept)
+__host__ __device__ constexpr bool thin_serves(int E, int n) { return E > 64 && (n <= 1024 || (n <= 2048 && E > 128)); }
+
+template <int WE>
+int launch_thin(const void* x, const void* w, const float* bias, const moe_router_params& p, int32_t* idx, float* tw,
+                float* lo, hipStream_t st) {
+    if (p.n_tokens <= 1024) return launch_thin_as<WE, 3>(x, w, bias, p, idx, tw, lo, st);
+    return launch_thin_as<WE, 2>(x, w, bias, p, idx, tw, lo, st);
+}
+
 template <int EBW>
 int launch_pairs(const void* x, const void* w, const float* bias, const moe_router_params& p, int32_t* idx, float* tw,
                  float* lo, hipStream_t st) {
@@ -692,10 +880,12 @@ extern "C" int moe_router_rmsnorm(const void* x, const void* norm_weight, float 
     MOE_REQUIRE(norm_weight && x_norm, "moe_router_rmsnorm: NULL norm weight or output");
     MOE_REQUIRE(x_norm != x, "moe_router_rmsnorm: x_norm must not alias x (rows are read twice)");
     MOE_REQUIRE(eps >= 0.0f, "moe_router_rmsnorm: eps %g < 0", (double)eps);
-    if (params != nullptr && params->n_experts <= 32) {
+    if (params != nullptr && (params->n_experts <= 32 ||
+                              thin_serves(params->n_experts, params->n_tokens))) {
         // Few experts: a launch is short chains of small MFMAs on few waves, with nothing to hide the
         // per-workgroup pre-pass behind (Mixtral-8x7B, 16384 tokens: 0.149 ms fused against 0.088 +
-        // 0.045 ms).  The norm kernel followed by the plain router gives the same bits.
+        // 0.045 ms).  Few tokens and many experts: the engine whose waves run without a common stage has no
+        // place for the pre-pass either.  The norm kernel followed by the plain router gives the same bits.
         int rc = moe_rmsnorm(x, norm_weight, eps, params->n_tokens, params->hidden, x_norm, stream);
         if (rc != MOE_OK) return rc;
         return route(x_norm, w_gate, bias, params, topk_idx, topk_w, logits_out, NormArgs{nullptr, 0.0f, nullptr}, stream);
@@ -742,15 +932,19 @@ int route(const void* x, const void* w_gate, const float* bias, const moe_router
     //   64 experts    4096 tokens: 16x16 0.040, 64x4 0.097;  24576: 0.122, 0.148;  32768: 0.157, 0.153;
     //                 131072: 64x4 0.45, 32x32 0.43
     //   8 experts    32768 tokens: 16x16 0.093, 64x4 0.104;  65536: 0.174, 0.144
-    //   160 experts   1024 tokens: 4x64 0.115, 16x16 0.131, 64x4 0.335;  8192: 16x16 0.250, 32x32 0.468;
-    //                 12288: 0.374, 0.479
-    //   256 experts   1024 tokens: 4x64 0.165, 16x16 0.231, 64x4 0.583;  8192: 16x16 0.519, 32x32 0.657;
-    //                 12288: 0.775, 0.683
+    //   160 experts   1024 tokens: 16x16 0.131, 64x4 0.335;  8192: 16x16 0.250, 32x32 0.468;  12288: 0.374, 0.479
+    //   256 experts   1024 tokens: 16x16 0.231, 64x4 0.583;  8192: 16x16 0.519, 32x32 0.657;  12288: 0.775, 0.683
+    //   (4 x 64, the layout for the fewest tokens, is router_thin_kernel's: see thin_serves)
     // up to 16 experts and few tokens: a lane per (token, expert) pair
     // measured (us, h = 4096; pairs / 4x4 engine): 8 experts 256 tokens 35 / 50, 8192: 42 / 53, 16384: 58 / 61,
     // 32768: 122 / 89; 16 experts 4096 tokens: 41 / 50, 8192: 81 / 53
     if (E <= 8 && n <= 8192 && !nrm.w) return launch_pairs<8>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
     if (E <= 16 && n <= 4096 && !nrm.w) return launch_pairs<16>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    if (thin_serves(E, n) && !nrm.w) {          // 4 or 8 tokens per workgroup, a wave alone per 64 experts
+        if (E <= 128) return launch_thin<2>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+        if (E <= 192) return launch_thin<3>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+        return launch_thin<4>(x, w_gate, bias, p, topk_idx, topk_w, logits_out, st);
+    }
     if (E <= 64) {
         if (n <= (E <= 32 ? 32768 : 24576)) {   // 16 tokens per workgroup, 16 experts per wave
             if (E <= 16) MOE_ROUTE(true, 4, 1, 1, 1, 16);
@@ -768,10 +962,6 @@ int route(const void* x, const void* w_gate, const float* bias, const moe_router
         }
         if (E <= 32) MOE_ROUTE(false, 16, 1, 1, 4, 32);
         MOE_ROUTE(false, 16, 1, 2, 2, 64);
-    }
-    if (n <= 1024 && E > 128) {                 // 4 tokens per workgroup, 64 experts per wave
-        if (E <= 192) MOE_ROUTE(true, 1, 1, 3, 1, 64);
-        MOE_ROUTE(true, 1, 1, 4, 1, 64);
     }
     if (n <= 8192) {                            // 16 tokens per workgroup, 16 experts per wave
         if (E <= 96) MOE_ROUTE(true, 4, 1, 6, 1, 64);

@@ -128,7 +128,8 @@ def test_every_expert_count_bracket(E):
     where the count allows groups, sigmoid group-limited routing; logits, indices and weights
     bit-for-bit.  The token count picks the logit engine and its block layout inside a bracket:
     150 tokens (full tiles and a ragged one) the vector-ALU engine with a lane per (token, expert) pair up to
-    16 experts, above that the 4x4 MFMA engine with 16 tokens per workgroup, or with 4 above 128 experts; 4100 tokens (more than 128 experts) 16 per workgroup; 8200 tokens
+    16 experts, above that the 4x4 MFMA engine with 16 tokens per workgroup, above 64 experts the engine whose waves
+    run without a common stage (4 tokens per workgroup); 4100 tokens (more than 128 experts) 16 per workgroup; 8200 tokens
     (more than 64 experts) the 32x32 MFMA engine (129 to 208 experts: with extra 4-expert groups per wave); up to 64 experts 33000 tokens the 4x4 engine with
     64 tokens per workgroup and 65600 the 32x32 engine (always 4x4 up to 16 experts)."""
     print(f"router bracket E={E}", flush=True)
@@ -158,12 +159,32 @@ def test_every_expert_count_bracket(E):
             assert np.array_equal(w.view(np.uint32), ow.view(np.uint32)), (E, n, spec.method)
 
 
+@pytest.mark.parametrize("E,n", [(96, 37), (256, 1024), (160, 1500), (256, 2048), (200, 1025)])
+def test_barrier_free_engine_stage_counts(E, n):
+    """More than 64 experts and few tokens: every wave streams its 64 gate rows through LDS buffers of its own, three
+    of them up to 1024 tokens (the k loop unrolled by six stages of 64) and two up to 2048 tokens above 128 experts
+    (unrolled by two).  Hidden sizes that leave 0 ... 5 whole stages after the unrolled loop, with and without a last
+    stage of fewer than 64 k, and sizes below one stage; bit for bit against the oracle."""
+    spec = O.RouterSpec.deepseek_v3(E, 6, 4, 2, True, 2.5) if E % 4 == 0 else O.RouterSpec.deepseek_v2(E, 6, "greedy")
+    for h in (8, 56, 64, 72, 128, 384, 392, 448, 456, 576, 640, 704, 760):
+        print(f"barrier-free engine E={E} n={n} h={h}", flush=True)
+        g = torch.Generator().manual_seed(h + E)
+        x = torch.randn(n, h, generator=g).to(torch.bfloat16)
+        wg = (torch.randn(E, h, generator=g) * 0.1).to(torch.bfloat16)
+        bias = (torch.randn(E, generator=g) * 0.01) if spec.method == "noaux_tc" else None
+        idx, w, lg = gpu_router(x, wg, bias, spec)
+        oi, ow, ol = O.router(bits(x), bits(wg), None if bias is None else bias.numpy(), spec)
+        assert np.array_equal(lg.view(np.uint32), ol.view(np.uint32)), (E, n, h)
+        assert np.array_equal(idx, oi), (E, n, h)
+        assert np.array_equal(w.view(np.uint32), ow.view(np.uint32)), (E, n, h)
+
+
 def test_router_random_shapes_at_switch_points():
     """Seeded random rules (expert count, top-k, family, groups) at token counts on both sides of
     every switch point of the logit engine's dispatch, bit-for-bit against the oracle."""
     import random
     rng = random.Random(7)
-    edges = [1, 3, 4, 5, 7, 8, 9, 15, 16, 17, 63, 64, 65, 1023, 1024, 1025, 4095, 4096, 4097, 8191, 8192, 8193, 24576, 24577, 32768,
+    edges = [1, 3, 4, 5, 7, 8, 9, 15, 16, 17, 63, 64, 65, 1023, 1024, 1025, 2047, 2048, 2049, 4095, 4096, 4097, 8191, 8192, 8193, 24576, 24577, 32768,
              32769, 65536, 65537]
     for it in range(56):
         E = rng.choice([1, 3, 7, 8, 9, 16, 20, 31, 32, 40, 50, 64, 72, 96, 120, 129, 160, 190, 208, 240, 256])
