@@ -20,7 +20,8 @@ def rand_idx(n, k, E, seed, skew=False):
 
 
 @pytest.mark.parametrize("n,k,E", [(1, 1, 1), (7, 2, 8), (300, 6, 64), (2048, 8, 256), (5000, 6, 160),
-                                   (4097, 2, 8), (33, 8, 256)])
+                                   (4097, 2, 8), (33, 8, 256),
+                                   (1536, 8, 256), (1537, 8, 256), (767, 16, 200)])   # either side of the one-workgroup form's 12288 entries
 @pytest.mark.parametrize("skew", [False, True])
 def test_dispatch_bit_exact(n, k, E, skew):
     from moe_gen_amd import ops
