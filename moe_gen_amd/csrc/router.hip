@@ -241,7 +241,7 @@ __device__ void route_token(const float* row, const float* __restrict__ bias, co
 //  SMALL == true : v_mfma_f32_4x4x1_16b_f32: 16 independent 4x4 blocks in 8 cycles, so nothing is
 //                  padded to 32 experts and the sequential-in-k dependency chain is 8x shorter.  The
 //                  blocks are TG groups of 4 tokens x 16/TG groups of 4 experts: TG = 16 is 64 tokens
-//                  x 4 experts per instruction, TG = 4 is 16 x 16, TG = 1 is 4 x 64; a workgroup owns
+//                  x 4 experts per instruction, TG = 4 is 16 x 16 (4 x 64 is router_thin_kernel's); a workgroup owns
 //                  4*TG tokens.  NEB instructions per k and wave, WE waves along experts.  Used for
 //                  E <= 16 (Mixtral's 8 experts) and for few tokens: a handful of workgroups cannot hide
 //                  the 64-cycle latency of the 32x32 chain, and fewer tokens per workgroup spread the
