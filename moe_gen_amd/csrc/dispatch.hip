@@ -168,19 +168,24 @@ __global__ __launch_bounds__(64 * SMALL_WAVES) void dispatch_small(const int32_t
                                                                    int32_t* __restrict__ offsets,
                                                                    int32_t* __restrict__ perm, int32_t* __restrict__ pos,
                                                                    int32_t* __restrict__ row_map, int k) {
+    constexpr int IT = SMALL_MAX / (SMALL_WAVES * 64);   // 64-entry steps of a wave's slice, at most
     __shared__ int whist[SMALL_WAVES][MAX_E];
     __shared__ int wtot[4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int slice = (nk + SMALL_WAVES * 64 - 1) / (SMALL_WAVES * 64) * 64;
     const int wbase = wave * slice;
+    // the lane's entries of the slice, all requested at once (both passes use them: a load per step would put the
+    // memory latency into every step); -1 marks an entry past the list or an id outside [0, E)
+    int ev[IT];
+#pragma unroll
+    for (int it = 0; it < IT; ++it) ev[it] = idx[min(wbase + 64 * it + lane, nk - 1)];
     for (int e = tid; e < SMALL_WAVES * MAX_E; e += 64 * SMALL_WAVES) (&whist[0][0])[e] = 0;
     __syncthreads();
-    for (int i = lane; i < slice; i += 64) {
-        const int g = wbase + i;
-        if (g < nk) {
-            const int e = idx[g];
-            if ((unsigned)e < (unsigned)E) atomicAdd(&whist[wave][e], 1);
-        }
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        const int g = wbase + 64 * it + lane;
+        if (64 * it >= slice || g >= nk || (unsigned)ev[it] >= (unsigned)E) ev[it] = -1;
+        if (ev[it] >= 0) atomicAdd(&whist[wave][ev[it]], 1);
     }
     __syncthreads();
     int cv = 0, inc = 0;
@@ -213,12 +218,13 @@ __global__ __launch_bounds__(64 * SMALL_WAVES) void dispatch_small(const int32_t
     }
     __syncthreads();
     int* cur = whist[wave];
-    for (int i0 = 0; i0 < slice; i0 += 64) {
-        const int g = wbase + i0 + lane;
-        const bool in_list = g < nk;
-        const int e = in_list ? idx[g] : 0;
-        const bool ok = in_list && (unsigned)e < (unsigned)E;
-        if (in_list && !ok) pos[g] = -1;       // as in rank_scatter: no sorted row, the combine skips the slot
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        if (64 * it >= slice) break;
+        const int g = wbase + 64 * it + lane;
+        const int e = ev[it];
+        const bool ok = e >= 0;
+        if (g < nk && !ok) pos[g] = -1;        // as in rank_scatter: no sorted row, the combine skips the slot
         uint64_t peers = __ballot(ok);
 #pragma unroll
         for (int b = 0; b < 8; ++b) {

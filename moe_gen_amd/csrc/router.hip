@@ -705,13 +705,13 @@ __global__ __launch_bounds__(64 * WE, NBUF == 2 ? 2 : 1) void router_thin_kernel
     };
     // token values straight from memory into the broadcast layout: register g of a stage holds, in lanes
     // 4b .. 4b+3, element 16 g + b of the 4 tokens (one 2-byte load per lane and 16 k), widened when its 16 k come up
-    const uint16_t* const xlane = x + (size_t)min(t0 + (lane & 3), n - 1) * h + (lane >> 2);
+    const uint16_t* const xrow = x + (size_t)min(t0 + (lane & 3), n - 1) * h;
     uint32_t xr[2][4];
-    auto load_x = [&](int set, int st) {
+    auto load_x = [&](int set, int st) {       // (elements past h are never multiplied: any address inside the row will do)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            const int k = st * KC + 16 * g;
-            xr[set][g] = xlane[k + (lane >> 2) < h ? k : 0];
+            const int k = st * KC + 16 * g + (lane >> 2);
+            xr[set][g] = xrow[k < h ? k : 0];
         }
     };
 
