@@ -723,17 +723,19 @@ __global__ __launch_bounds__(64 * WE, NBUF == 2 ? 2 : 1) void router_thin_kernel
     auto wf = [](const u32x4& v, int j) {      // element j of 8 bf16 as fp32
         return __uint_as_float((j & 1) ? (v[j >> 1] & 0xffff0000u) : (v[j >> 1] << 16));
     };
-    // Stage st; the register set st & 1 and the buffers are literals at every call site.  The loads of stage
-    // st + NBUF - 1 (weights) and st + 2 (tokens) leave first, then the wait that lets the vector-memory operations
-    // younger than the DMA of stage st stay in flight (per stage ahead 8 DMA and 4 token loads).
+    // Stage st; the register set st & 1 and the buffers are literals at every call site.  The DMA of stage
+    // st + NBUF - 1 leaves first, then the wait for the DMA of stage st.  Its count is the DMA instructions issued
+    // since -- 8 per stage ahead -- and nothing else: the token loads sit behind the wait in program order, but the
+    // compiler may place a register load on either side of it, and every one that is in the window only makes the
+    // wait stricter (the oldest operations in the window are token loads of a stage ago, long complete).
     auto stage = [&](int st, int set, const uint8_t* wb, uint8_t* wb_refill, int nch) {
         uint32_t xs[4];
 #pragma unroll
         for (int g = 0; g < 4; ++g) xs[g] = xr[set][g];
-        load_x(set, min(st + 2, nstage - 1));
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the reads of stage st - 1, a stage old, before their buffer is refilled
         dma_w(wb_refill, min(st + NBUF - 1, nstage - 1));
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NBUF - 1) * (8 + 4)) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NBUF - 1) * 8) : "memory");
+        load_x(set, min(st + 2, nstage - 1));            // (tokens of stage st + 2 into the set that held stage st)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             if (2 * g >= nch) break;
@@ -765,8 +767,8 @@ __global__ __launch_bounds__(64 * WE, NBUF == 2 ? 2 : 1) void router_thin_kernel
         }
     } else {
         load_x(0, 0);
-        dma_w(wb0, 0);
         load_x(1, min(1, nstage - 1));
+        dma_w(wb0, 0);
         dma_w(wb1, min(1, nstage - 1));
         for (; st + 6 <= nfull; st += 6) {
             stage(st, 0, wb0, wb2, 8);
