@@ -261,7 +261,8 @@ int moe_rmsnorm(const void* x, const void* weight, float eps, int32_t n_tokens, 
  * its tokens (moe_rmsnorm's summation order), normalises every chunk on its way to the matrix
  * cores, xn = bf16(weight * bf16(f32(x) * rstd)), and writes the normalised rows once to x_norm
  * for the expert GEMMs.  Results (x_norm, indices, weights, logits) are bit-identical to
- * moe_rmsnorm followed by moe_router (with 32 experts or fewer, where the fused form does not pay,
+ * moe_rmsnorm followed by moe_router (with 32 experts or fewer, and with more than 64 experts and a
+ * small batch -- up to 1024 tokens, 2048 above 128 experts --, where the fused form does not pay,
  * the call is those two launches).
  *   x           device bf16 [n, h]  raw hidden states
  *   norm_weight device bf16 [h]
