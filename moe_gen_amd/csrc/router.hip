@@ -815,16 +815,18 @@ int launch_thin_as(const void* x, const void* w, const float* bias, const moe_ro
     MOE_HIP_CHECK(hipGetLastError());
     return MOE_OK;
 }
-// Which calls the engine above serves.  On this chip a 4x4x1 MFMA keeps its wave for about 16 cycles whether or not
-// the next one depends on it, and two waves of a SIMD share the matrix core (two chains in one wave took 1.75 times
-// as long as one, two workgroups per CU 1.5 times), so once every CU has two workgroups the engines with more tokens
-// per instruction win.  Up to 1024 tokens: one workgroup per CU, three buffers.  Up to 2048 tokens and above 128
-// experts: two workgroups per CU, two buffers.  Measured (us, router_kernel -> this; h = 7168 / 5120):
+// Which calls the engine above serves.  In registers a 4x4x1 MFMA issues every 8.6 cycles, every 15.5 when it
+// depends on the one before; in this kernel a second, independent chain per wave (8 tokens per workgroup) still took
+// 1.75 times as long as one, and two workgroups per CU take 1.5 times as long as one, so once every CU has two
+// workgroups the engines with more tokens per instruction win.  Up to 1024 tokens: one workgroup per CU, three
+// buffers.  Up to 2048 tokens and above 128 experts: two workgroups per CU, two buffers.  Measured (us,
+// router_kernel -> this; h = 7168 / 5120):
 //   256 experts:  64 ... 1024 tokens 165 ... 178 -> 97 ... 106;  2048 tokens 232 -> 171;  3072: 235 against 258
 //   160 experts:  1024 tokens 96 -> 78;  2048 tokens 134 -> 118;  3072: 138 against 153
 //   128 experts:  1024 tokens 91 -> 77;  2048: 98 against 114
-// (a 16-token form on v_mfma_f32_16x16x1_4b_f32, 32 cycles per k by the book, ran at 77: 304 us at 4096 tokens of
-// 256 experts against 248; with two workgroups per CU 410 against 474 at 8192 tokens and behind again from 12288: not kept)
+// (a 16-token form on v_mfma_f32_16x16x1_4b_f32, 32 cycles per instruction in registers, ran at 77 per k: 304 us at
+// 4096 tokens of 256 experts against 248; with two workgroups per CU 410 against 474 at 8192 tokens and behind again
+// from 12288: not kept)
 __host__ __device__ constexpr bool thin_serves(int E, int n) { return E > 64 && (n <= 1024 || (n <= 2048 && E > 128)); }
 
 template <int WE>
